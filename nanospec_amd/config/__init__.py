@@ -1,0 +1,9 @@
+from .llama import LlamaConfig
+from .registry import architectures, load_config, register_architecture, resolve
+from .spec import (AttentionSpec, LayerCall, ModelSpec, NoPositionSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec,
+                   SwiGLUSpec)
+
+__all__ = [
+    "LlamaConfig", "architectures", "load_config", "register_architecture", "resolve", "AttentionSpec", "LayerCall",
+    "ModelSpec", "NoPositionSpec", "PreNormBlockSpec", "RMSNormSpec", "RopeSpec", "SwiGLUSpec",
+]

@@ -1,0 +1,276 @@
+// Soft-max attention over the paged bfloat16 cache on the matrix cores, for prefill portions and for
+// decode, compiled for one head size (NS_HEAD_DIM, a multiple of 16 up to 256).
+//
+// One wave owns one tile of 16 "columns".  A column is a (query token, query head) pair of one
+// request and one key/value head: hp consecutive heads of the group times 16/hp consecutive tokens.
+// Prefill portions run with hp = 1 (16 tokens of one head), decode with hp = the group size, so
+// that all query heads that share a key/value head share each load of it.
+// (reference: model/attention.py:22-43 for what is computed, :86-101 for the two modes)
+//
+// Everything is kept transposed so that a column is always lane % 16:
+//   S^T[key][col] = K[key][:] . Q[col][:]        A = K tile (rows = keys, straight from the page),
+//                                                B = Q^T (lane holds 8 channels of its column)
+//   soft-max over keys: the 8 keys a lane holds, then across the 4 lane groups (xor 16, 32)
+//   O^T[ch][col] += V^T[ch][key] . P^T[key][col]  A = V^T tile, which the cache stores as
+//                                                [page][kv head][channel][token]: 4 consecutive
+//                                                tokens per 8-byte load; B = P^T is exactly the
+//                                                layout S^T came out in.
+// The running maximum, the running sum and the output accumulators of a column therefore live in
+// the lanes of that column and are rescaled without any exchange.
+//
+// Query at position p sees keys max(0, p - window + 1) .. p.  Scores, soft-max and sums are 32-bit.
+// With splits > 1 the keys of a tile are cut into `splits` contiguous ranges of whole 32-key blocks;
+// each range writes its un-normalised output, maximum and sum, and ns_attn_mfma_reduce joins them.
+#include "common.h"
+
+#ifndef NS_HEAD_DIM
+#error "compile with -DNS_HEAD_DIM=<multiple of 16>"
+#endif
+constexpr int HD = NS_HEAD_DIM;
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
+constexpr int DT = HD / 16;         // 16-channel tiles of the output
+constexpr bool WIDE = HD % 32 == 0;  // q.k with the k=32 instruction, else with k=16
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+struct AttnParams {
+  bf16_t* out;        // [tokens, heads, HD]
+  float* part_o;      // [tokens * heads, splits, HD]   (splits > 1)
+  float* part_ml;     // [tokens * heads, splits, 2]
+  const bf16_t* q;    // row t at q + t * q_stride, head h at + h * HD
+  const bf16_t* k_cache;
+  const bf16_t* v_cache;
+  const int* tile_req;  // [n_tiles] request of the tile
+  const int* tile_t0;   // [n_tiles] first token of the tile within the request's tokens of this step
+  const int* qo_indptr;  // [requests + 1]
+  const int* kv_lens;    // [requests] keys after this step's tokens are written
+  const int* block_table;
+  int q_stride, table_stride, n_tiles, heads, kv_heads, page_size, hp, splits, window;
+  float scale_log2;  // softmax scale * log2(e)
+};
+
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+__global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int G = a.heads / a.kv_heads;
+  const int hblks = (G + a.hp - 1) / a.hp;
+  const int ny = a.kv_heads * hblks;
+  const long item = (long)blockIdx.x * 4 + wave;
+  if (item >= (long)a.n_tiles * a.splits * ny) return;
+  const int y = (int)(item % ny);
+  const long ts = item / ny;
+  const int split = (int)(ts % a.splits), tile = (int)(ts / a.splits);
+  const int kvh = y / hblks, hblk = y % hblks;
+  const int b = a.tile_req[tile], t0 = a.tile_t0[tile];
+  const int q0 = a.qo_indptr[b], n = a.qo_indptr[b + 1] - q0, kv_len = a.kv_lens[b];
+  const int* table = a.block_table + (size_t)b * a.table_stride;
+  const int ps = a.page_size;
+
+  // this lane's column
+  const int ti = t0 + c / a.hp;
+  const int hin = hblk * a.hp + c % a.hp;
+  const bool col_ok = ti < n && hin < G;
+  const int head = kvh * G + (col_ok ? hin : 0);
+  const int pos = col_ok ? kv_len - n + ti : -1;
+  const int lo = (col_ok && a.window > 0) ? max(0, pos - a.window + 1) : 0;
+  const int whi = wave_max_i(pos) + 1;                    // keys [wlo, whi) are seen by some column
+  const int wlo = wave_min_i(col_ok ? lo : 0x7fffffff);
+  if (whi <= 0) return;
+
+  int kb0 = wlo / 32, kb1 = (whi + 31) / 32;
+  if (a.splits > 1) {
+    const int per = (kb1 - kb0 + a.splits - 1) / a.splits;
+    kb0 = kb0 + split * per;
+    kb1 = min(kb1, kb0 + per);
+  }
+
+  // Q^T fragments of this lane's column
+  const bf16_t* qrow = a.q + (size_t)(q0 + (col_ok ? ti : 0)) * a.q_stride + head * HD;
+  bf16x8 qw[WIDE ? HD / 32 : 1];
+  s16x4 qn[WIDE ? 1 : HD / 16];
+  if (WIDE) {
+#pragma unroll
+    for (int i = 0; i < HD / 32; ++i) {
+      qw[i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32 + g * 8);
+      if (!col_ok) qw[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) {
+      qn[i] = *reinterpret_cast<const s16x4*>(qrow + i * 16 + g * 4);
+      if (!col_ok) qn[i] = s16x4{0, 0, 0, 0};
+    }
+  }
+
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+  const int qlo = wlo & ~3, qhi = (whi - 1) & ~3;  // first and last 4-key group that holds a seen key
+
+  for (int kb = kb0; kb < kb1; ++kb) {
+    const int key_base = kb * 32;
+    // ---- S^T = K . Q^T for two tiles of 16 keys
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);  // keep the address inside held pages
+      const int page = table[key / ps];
+      const bf16_t* krow = a.k_cache + (((size_t)page * ps + key % ps) * a.kv_heads + kvh) * HD;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      if (WIDE) {
+#pragma unroll
+        for (int i = 0; i < HD / 32; ++i)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + i * 32 + g * 8), qw[i], acc, 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int i = 0; i < HD / 16; ++i)
+          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s16x4*>(krow + i * 16 + g * 4), qn[i], acc, 0, 0, 0);
+      }
+      s[t] = acc;
+    }
+    // ---- mask, running maximum, probabilities.  s[t][j] is key key_base + 16 t + 4 g + j of column c.
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int key = key_base + t * 16 + g * 4 + j;
+        const float v = (key >= lo && key <= pos) ? s[t][j] * a.scale_log2 : -INFINITY;
+        s[t][j] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(m - m_safe);
+    m = m_new;
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float p = exp2f(s[t][j] - m_safe);
+        psum += p;
+        pf[t * 4 + j] = (bf16_t)p;
+      }
+    lsum = lsum * alpha + psum;
+    // ---- O^T = O^T * alpha + V^T . P^T.  Slot 8 g + j of the instruction holds key key_base + 4 g + j
+    //      for j < 4 and key_base + 16 + 4 g + (j - 4) for j >= 4, in both operands.
+    const int k0 = min(max(key_base + g * 4, qlo), qhi);
+    const int k1 = min(max(key_base + 16 + g * 4, qlo), qhi);
+    const size_t v0 = ((size_t)table[k0 / ps] * a.kv_heads + kvh) * HD * ps + k0 % ps;
+    const size_t v1 = ((size_t)table[k1 / ps] * a.kv_heads + kvh) * HD * ps + k1 % ps;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const size_t ch = (size_t)(dt * 16 + c) * ps;
+      const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(a.v_cache + v0 + ch);
+      const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(a.v_cache + v1 + ch);
+      const bf16x8 vf = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+    }
+  }
+
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  if (!col_ok) return;
+  // o[dt][j] is channel 16 dt + 4 g + j of column c
+  const size_t col = (size_t)(q0 + ti) * a.heads + head;
+  if (a.splits == 1) {
+    const float inv = 1.f / lsum;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x4 r = {(bf16_t)(o[dt][0] * inv), (bf16_t)(o[dt][1] * inv), (bf16_t)(o[dt][2] * inv), (bf16_t)(o[dt][3] * inv)};
+      *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
+    }
+  } else {
+    float* po = a.part_o + (col * a.splits + split) * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
+    if (g == 0) {
+      a.part_ml[(col * a.splits + split) * 2] = m;
+      a.part_ml[(col * a.splits + split) * 2 + 1] = lsum;
+    }
+  }
+}
+
+// out[col] = sum_s o_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*), m* = max_s m_s; splits are joined in order.
+// One workgroup per (tile, head): it joins the columns of that head for the tile's tokens.
+__global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
+                                                         const float* __restrict__ part_ml,
+                                                         const int* __restrict__ tile_req, const int* __restrict__ tile_t0,
+                                                         const int* __restrict__ qo_indptr, int heads, int hp, int splits) {
+  const int b = tile_req[blockIdx.x], t0 = tile_t0[blockIdx.x], head = blockIdx.y;
+  const int q0 = qo_indptr[b], n = qo_indptr[b + 1] - q0;
+  const int t1 = min(n, t0 + 16 / hp);
+  for (int ti = t0; ti < t1; ++ti) {
+    const size_t col = (size_t)(q0 + ti) * heads + head;
+    const float* ml = part_ml + col * splits * 2;
+    float mstar = -INFINITY;
+    for (int s = 0; s < splits; ++s) mstar = fmaxf(mstar, ml[s * 2]);
+    float l = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = ml[s * 2];
+      if (ms != -INFINITY) l += ml[s * 2 + 1] * exp2f(ms - mstar);
+    }
+    for (int d = threadIdx.x; d < HD; d += 64) {
+      float acc = 0.f;
+      for (int s = 0; s < splits; ++s) {
+        const float ms = ml[s * 2];
+        if (ms != -INFINITY) acc += part_o[(col * splits + s) * HD + d] * exp2f(ms - mstar);
+      }
+      out[col * HD + d] = (bf16_t)(acc / l);
+    }
+  }
+}
+
+extern "C" int ns_attn_mfma_head_dim() { return HD; }
+
+// Workspace, when splits > 1: part_o holds tokens*heads*splits*HD floats, part_ml tokens*heads*splits*2.
+extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
+                            const void* v_cache, const int* tile_req, const int* tile_t0, const int* qo_indptr,
+                            const int* kv_lens, const int* block_table, int table_stride, int n_tiles, int n_tokens,
+                            int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale,
+                            hipStream_t stream) {
+  if (n_tiles <= 0 || n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || (page_size & 3) ||
+      window < 0 || splits < 1 || (q_stride & 7))
+    return NS_ERR_BAD_ARG;
+  if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
+  if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
+  AttnParams a;
+  a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
+  a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
+  a.tile_req = tile_req; a.tile_t0 = tile_t0; a.qo_indptr = qo_indptr; a.kv_lens = kv_lens; a.block_table = block_table;
+  a.q_stride = q_stride; a.table_stride = table_stride; a.n_tiles = n_tiles; a.heads = heads; a.kv_heads = kv_heads;
+  a.page_size = page_size; a.hp = hp; a.splits = splits; a.window = window;
+  a.scale_log2 = scale * 1.4426950408889634f;
+  const int G = heads / kv_heads;
+  const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);
+  const long blocks = (items + 3) / 4;
+  if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
+  attn_mfma_kernel<<<(unsigned)blocks, 256, 0, stream>>>(a);
+  int st = ns_launch_status();
+  if (st != NS_OK || splits == 1) return st;
+  if (heads > 65535) return NS_ERR_BAD_ARG;
+  attn_reduce_kernel<<<dim3(n_tiles, heads), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml, tile_req,
+                                                             tile_t0, qo_indptr, heads, hp, splits);
+  return ns_launch_status();
+}

@@ -1,0 +1,57 @@
+"""A bump allocator for the intermediates of one step.
+
+Every buffer a part needs between kernels comes from here, so a step allocates nothing from the
+framework's general allocator once the arena has grown to its working size, and a captured graph
+owns an arena of fixed size whose addresses never change.  ``mark``/``release`` let a layer hand its
+buffers back for the next layer.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+_ALIGN = 256
+
+
+class Arena:
+    def __init__(self, device, nbytes: int = 0, fixed: bool = False) -> None:
+        self.device, self.fixed = device, fixed
+        self._chunks: list[torch.Tensor] = []
+        self._cur, self._off = -1, 0
+        self._high = 0  # bytes one step needed at most, over all chunks
+        if nbytes:
+            self._chunks.append(torch.empty(nbytes, dtype=torch.uint8, device=device))
+            self._cur = 0
+
+    def take(self, shape, dtype) -> torch.Tensor:
+        shape = tuple(int(s) for s in shape)
+        nbytes = max(1, math.prod(shape)) * torch.empty(0, dtype=dtype).element_size()
+        need = -(-nbytes // _ALIGN) * _ALIGN
+        while self._cur < 0 or self._off + need > self._chunks[self._cur].numel():
+            if self._cur + 1 < len(self._chunks):
+                self._cur, self._off = self._cur + 1, 0
+                continue
+            if self.fixed:
+                raise RuntimeError(f"a fixed arena of {sum(c.numel() for c in self._chunks)} bytes is exhausted")
+            size = max(need, 2 * sum(c.numel() for c in self._chunks), 1 << 20)
+            self._chunks.append(torch.empty(size, dtype=torch.uint8, device=self.device))
+            self._cur, self._off = len(self._chunks) - 1, 0
+        chunk = self._chunks[self._cur]
+        out = chunk[self._off : self._off + nbytes].view(dtype).view(shape)
+        self._off += need
+        return out
+
+    def mark(self) -> tuple[int, int]:
+        return self._cur, self._off
+
+    def release(self, mark: tuple[int, int]) -> None:
+        self._cur, self._off = mark
+
+    def reset(self) -> None:
+        """Start of a step.  Several chunks mean the arena grew during the last step: merge them."""
+        if len(self._chunks) > 1 and not self.fixed:
+            total = sum(c.numel() for c in self._chunks)
+            self._chunks = [torch.empty(total, dtype=torch.uint8, device=self.device)]
+        self._cur, self._off = (0, 0) if self._chunks else (-1, 0)

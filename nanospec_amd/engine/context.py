@@ -1,0 +1,148 @@
+"""One step's batch as the parts see it: flat token arrays, per-request arrays, block tables per cache
+group and the tile lists of the attention kernels, all views of ONE int32 buffer that is filled on the
+host and copied to the device in one piece.
+
+Layout of the batch (reference: kv/cache.py:42-61,125-157 builds the same facts as qo_indptr /
+kv_indptr / kv_indices / kv_last_page_len / positions / slots):
+    token_ids[N] positions[N] token_req[N]        per token; token_req = index of its request in the batch
+    qo_indptr[B+1] kv_lens[B] state_slots[B]      per request; kv_lens counts the keys after this step
+    want_rows[R]                                  token rows whose logits are wanted
+    chunk tiles (tile_req, tile_t0)[Tc]           requests with more than one token, 16 tokens per tile
+    decode tiles (tile_req, tile_t0)[Td]          requests with exactly one token
+    block_table[g][B, P]                          page of positions [i*page, (i+1)*page), -1 if released
+Slots are not materialised: the kernels compute page and offset from the position and the block table.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+CHUNK_TILE = 16  # tokens per attention tile of a prompt portion
+
+
+def _pad4(n: int) -> int:
+    return -(-n // 4) * 4
+
+
+class BatchLayout:
+    """Offsets of the fields inside the int32 buffer for given sizes."""
+
+    def __init__(self, n_tokens: int, n_reqs: int, n_want: int, n_chunk_tiles: int, n_decode_tiles: int, n_groups: int,
+                 table_width: int) -> None:
+        self.N, self.B, self.R, self.Tc, self.Td, self.G, self.P = n_tokens, n_reqs, n_want, n_chunk_tiles, n_decode_tiles, n_groups, table_width
+        off = 0
+        self.fields = {}
+        for name, size in (("token_ids", n_tokens), ("positions", n_tokens), ("token_req", n_tokens), ("qo_indptr", n_reqs + 1),
+                           ("kv_lens", n_reqs), ("state_slots", n_reqs), ("want_rows", n_want), ("ctile_req", n_chunk_tiles),
+                           ("ctile_t0", n_chunk_tiles), ("dtile_req", n_decode_tiles), ("dtile_t0", n_decode_tiles)):
+            self.fields[name] = (off, size)
+            off += _pad4(max(size, 1))
+        self.table_off = []
+        for _ in range(n_groups):
+            self.table_off.append(off)
+            off += _pad4(max(n_reqs * table_width, 1))
+        self.total = off
+
+
+@dataclass
+class AttentionPlan:
+    tile_req: torch.Tensor
+    tile_t0: torch.Tensor
+    hp: int
+    splits: int
+    workspace: tuple | None
+
+
+class StepContext:
+    """Device views of one step's batch plus the arena; handed to every part."""
+
+    def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, fixed_splits: bool = False) -> None:
+        self.layout, self.arena = layout, arena
+        self.n_tokens, self.n_reqs = layout.N, layout.B
+        self.max_position, self.max_kv_len = max_position, max_kv_len
+        self.fixed_splits = fixed_splits
+        f = layout.fields
+
+        def view(name):
+            off, size = f[name]
+            return dev_buf[off : off + size]
+
+        self.token_ids, self.positions, self.token_req = view("token_ids"), view("positions"), view("token_req")
+        self.qo_indptr, self.kv_lens, self.state_slots = view("qo_indptr"), view("kv_lens"), view("state_slots")
+        self.want_rows = view("want_rows")
+        self._ctiles = (view("ctile_req"), view("ctile_t0"))
+        self._dtiles = (view("dtile_req"), view("dtile_t0"))
+        self.block_tables = [dev_buf[o : o + layout.B * layout.P].view(layout.B, layout.P) for o in layout.table_off]
+
+    def attention_plans(self, group: int, kv_heads: int, head_dim: int) -> list[AttentionPlan]:
+        """How the matrix-core attention kernel is launched for a mixer with ``group`` query heads per
+        key/value head: prompt portions as 16-token tiles of one head; decode rows with all heads of a
+        group in one tile and the keys cut into ranges so that the launch fills the GPU."""
+        plans = []  # made afresh per call: the workspace lives in the caller's arena scope
+        lay = self.layout
+        if lay.Tc:
+            plans.append(AttentionPlan(self._ctiles[0], self._ctiles[1], 1, 1, None))
+        if lay.Td:
+            hp = 1
+            while hp < min(group, 16):
+                hp *= 2
+            items = lay.Td * kv_heads * -(-group // hp)
+            splits = max(1, min(32, -(-1024 // items)))
+            if not self.fixed_splits:
+                splits = max(1, min(splits, -(-self.max_kv_len // 128)))
+            ws = None
+            if splits > 1:
+                cols = lay.N * kv_heads * group
+                ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
+            plans.append(AttentionPlan(self._dtiles[0], self._dtiles[1], hp, splits, ws))
+        return plans
+
+
+def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, slots, want_rows, tables: list[np.ndarray]) -> None:
+    """Write one batch into ``host`` (int32, at least layout.total long).  ``starts``/``lens``: first
+    position and token count per request; ``tables[g]``: int32 [B, P] block tables."""
+    f = layout.fields
+    B = layout.B
+    lens_a = np.asarray(lens, dtype=np.int32)
+    starts_a = np.asarray(starts, dtype=np.int32)
+    indptr = np.zeros(B + 1, dtype=np.int32)
+    np.cumsum(lens_a, out=indptr[1:])
+
+    def put(name, arr):
+        off, size = f[name]
+        host[off : off + size] = arr
+
+    put("token_ids", np.asarray(token_ids, dtype=np.int32))
+    req_of = np.repeat(np.arange(B, dtype=np.int32), lens_a)
+    put("token_req", req_of)
+    put("positions", np.arange(layout.N, dtype=np.int32) - indptr[req_of] + starts_a[req_of])
+    put("qo_indptr", indptr)
+    put("kv_lens", starts_a + lens_a)
+    put("state_slots", np.asarray(slots, dtype=np.int32))
+    if layout.R:
+        put("want_rows", np.asarray(want_rows, dtype=np.int32))
+    ct_req, ct_t0, dt_req = [], [], []
+    for b, n in enumerate(lens):
+        if n == 1:
+            dt_req.append(b)
+        else:
+            for t0 in range(0, n, CHUNK_TILE):
+                ct_req.append(b)
+                ct_t0.append(t0)
+    if layout.Tc:
+        put("ctile_req", np.asarray(ct_req, dtype=np.int32))
+        put("ctile_t0", np.asarray(ct_t0, dtype=np.int32))
+    if layout.Td:
+        put("dtile_req", np.asarray(dt_req, dtype=np.int32))
+        put("dtile_t0", np.zeros(len(dt_req), dtype=np.int32))
+    for g, off in enumerate(layout.table_off):
+        host[off : off + B * layout.P] = tables[g].reshape(-1)
+
+
+def count_tiles(lens) -> tuple[int, int]:
+    tc = sum(-(-n // CHUNK_TILE) for n in lens if n != 1)
+    td = sum(1 for n in lens if n == 1)
+    return tc, td

@@ -1,0 +1,264 @@
+"""The step function: a batch of (request, its next tokens) -> logits at the wanted places.
+
+``ModelRunner.step`` runs only the tokens it is given, as one batch, from the cache that earlier steps
+left: portions of prompts beside single decoded tokens, cut anywhere.  It reserves pages for the new
+tokens, builds the batch, runs the model and commits the new lengths.  Steps that hold one token per
+request replay a captured HIP graph when the model allows it.
+
+Reference: engine/engine.py:200-252 (rows per request, one forward, hidden states at the last rows)
+and model/llama.py:269-286 (logits only at the rows asked for).  Unlike the reference, prompts and
+decode rows share ONE forward, and a prompt may come in portions.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.storage import CacheStorage
+from ..kernels import ops
+from .arena import Arena
+from .context import BatchLayout, StepContext, count_tiles, fill_batch
+
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64)  # reference: engine/graphs.py:22
+PAD_REQUEST = "__pad__"
+
+
+@dataclass
+class StepEntry:
+    req_id: object
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)  # places among ``tokens`` whose logits are wanted
+
+
+class _DecodeGraph:
+    """One captured decode step for a bucket of ``size`` requests: static batch buffer, fixed arena,
+    logits for every row."""
+
+    def __init__(self, runner: "ModelRunner", size: int) -> None:
+        self.size = size
+        n_groups = len(runner.manager.groups)
+        self.layout = BatchLayout(size, size, size, 0, size, n_groups, runner.table_width)
+        dev = runner.device
+        self.dev_buf = torch.zeros(self.layout.total, dtype=torch.int32, device=dev)
+        self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.arena = Arena(dev)  # grows during the warm-up run, then stays as it is
+        self.logits: torch.Tensor | None = None
+        self.graph = None
+
+    def context(self, runner) -> StepContext:
+        return StepContext(self.layout, self.dev_buf, self.arena, max_position=0, max_kv_len=runner.table_width * runner.page_size,
+                           fixed_splits=True)
+
+
+class ModelRunner:
+    def __init__(self, model, manager: CacheManager, storage: CacheStorage, max_requests: int, table_width: int,
+                 use_graphs: bool = True) -> None:
+        self.model, self.manager, self.storage = model, manager, storage
+        self.device, self.dtype = model.device, model.dtype
+        self.page_size = manager.page_size
+        self.table_width = table_width  # pages per request a block table can name
+        self.max_requests = max_requests
+        self.stream = torch.cuda.Stream(device=self.device)
+        self.arena = Arena(self.device)
+        n_groups = len(manager.groups)
+        # host mirror of every live request's block tables, one row per state slot
+        self._tables = [np.full((manager.slots.num_slots, table_width), -1, dtype=np.int32) for _ in range(n_groups)]
+        self._mirrored = [[0] * manager.slots.num_slots for _ in range(n_groups)]
+        self._released = [[0] * manager.slots.num_slots for _ in range(n_groups)]
+        self._host = torch.zeros(1 << 14, dtype=torch.int32).pin_memory()
+        self._dev = torch.zeros(1 << 14, dtype=torch.int32, device=self.device)
+        self.use_graphs = bool(use_graphs and model.graph_safe)
+        self._graphs: dict[int, _DecodeGraph] = {}
+        self._pad_ready = False
+        self._staged: torch.cuda.Event | None = None
+        self.last_used_graph = False
+
+    # ------------------------------------------------------------------ requests
+
+    def admit(self, req_id) -> None:
+        rc = self.manager.admit(req_id)
+        for g in range(len(self._tables)):
+            self._mirrored[g][rc.slot] = 0
+            self._released[g][rc.slot] = 0
+        if self.storage.states:
+            with torch.cuda.stream(self.stream):
+                self.storage.reset_slot(rc.slot)
+
+    def release(self, req_id) -> None:
+        self.manager.release(req_id)
+
+    def _mirror(self, rc) -> None:
+        for g, table in enumerate(rc.tables):
+            if len(table) > self.table_width:
+                raise ValueError(f"request {rc.req_id!r} needs {len(table)} pages; block tables hold {self.table_width}")
+            row = self._tables[g][rc.slot]
+            have = self._mirrored[g][rc.slot]
+            if len(table) > have:
+                row[have : len(table)] = table[have:]
+                self._mirrored[g][rc.slot] = len(table)
+            first = rc.first_kept[g]
+            if first > self._released[g][rc.slot]:
+                row[self._released[g][rc.slot] : first] = -1
+                self._released[g][rc.slot] = first
+
+    # ------------------------------------------------------------------ the step
+
+    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+        """Run one batch.  -> float32 logits [number of wanted places, vocab] in the order of the entries
+        and of their ``want`` lists, or None if nothing is wanted."""
+        if not entries:
+            return None
+        vocab = self.model.spec.vocab_size
+        mgr = self.manager
+        seen = set()
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            if not e.tokens:
+                raise ValueError(f"request {e.req_id!r} brings no tokens")
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                raise ValueError(f"request {e.req_id!r} has a token id outside [0, {vocab})")
+            if any(not 0 <= w < len(e.tokens) for w in e.want):
+                raise ValueError(f"request {e.req_id!r} wants logits at a place it brings no token for")
+        # pages for everything first: running out leaves every request as it was
+        self._reserve_all(entries)
+        rcs = [mgr.get(e.req_id) for e in entries]
+        lens = [len(e.tokens) for e in entries]
+        starts = [rc.length for rc in rcs]
+        for rc in rcs:
+            self._mirror(rc)
+        n_want = sum(len(e.want) for e in entries)
+        caller = torch.cuda.current_stream(self.device)
+        self.stream.wait_stream(caller)  # whatever the caller still reads of the last step's results
+        if self._staged is not None:
+            self._staged.synchronize()  # the last batch has left the pinned staging buffers
+        with torch.cuda.stream(self.stream):
+            if self.use_graphs and all(n == 1 for n in lens) and n_want and self._bucket(len(entries)) is not None:
+                logits = self._step_graph(entries, rcs, starts)
+                self.last_used_graph = True
+            else:
+                logits = self._step_eager(entries, rcs, starts, lens, n_want)
+                self.last_used_graph = False
+        caller.wait_stream(self.stream)  # the caller's stream sees the logits
+        for e, rc in zip(entries, rcs):
+            mgr.commit(e.req_id, len(e.tokens))
+        return logits
+
+    def _reserve_all(self, entries) -> None:
+        mgr = self.manager
+        need = [0] * len(mgr.groups)
+        for e in entries:
+            for g, n in enumerate(mgr.pages_missing(e.req_id, len(e.tokens))):
+                need[g] += n
+        for g, n in enumerate(need):
+            if n > mgr.num_free(g):
+                from ..cache.pages import PoolExhausted
+
+                raise PoolExhausted(f"the step needs {n} more pages in group {mgr.groups[g].name!r}, {mgr.num_free(g)} free")
+        for e in entries:
+            mgr.reserve(e.req_id, len(e.tokens))
+
+    def _step_eager(self, entries, rcs, starts, lens, n_want):
+        n_tokens = sum(lens)
+        tc, td = count_tiles(lens)
+        max_kv = max(s + n for s, n in zip(starts, lens))
+        width = max(1, -(-max_kv // self.page_size))
+        layout = BatchLayout(n_tokens, len(entries), n_want, tc, td, len(self._tables), width)
+        if layout.total > self._host.numel():
+            size = 1 << (layout.total - 1).bit_length()
+            self._host = torch.zeros(size, dtype=torch.int32).pin_memory()
+            self._dev = torch.zeros(size, dtype=torch.int32, device=self.device)
+        slots = [rc.slot for rc in rcs]
+        token_ids = [t for e in entries for t in e.tokens]
+        want_rows, base = [], 0
+        for e, n in zip(entries, lens):
+            want_rows.extend(base + w for w in e.want)
+            base += n
+        tables = [t[slots, :width] for t in self._tables]
+        fill_batch(self._host.numpy(), layout, token_ids, starts, lens, slots, want_rows, tables)
+        self._dev[: layout.total].copy_(self._host[: layout.total], non_blocking=True)
+        self._staged = torch.cuda.Event()
+        self._staged.record(self.stream)
+        self.arena.reset()
+        ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv)
+        resid, delta = self.model.forward_hidden(ctx, self.storage.views)
+        if not n_want:
+            return None
+        return self.model.logits(ctx, resid, delta, ctx.want_rows)
+
+    # ------------------------------------------------------------------ graphs
+
+    def _bucket(self, n: int) -> int | None:
+        return next((b for b in GRAPH_BUCKETS if b >= n), None)
+
+    def _ensure_pad(self) -> None:
+        if not self._pad_ready:
+            self.manager.admit(PAD_REQUEST)
+            self.manager.reserve(PAD_REQUEST, 1)
+            self._mirror(self.manager.get(PAD_REQUEST))
+            self._pad_ready = True
+
+    def _fill_graph(self, g: _DecodeGraph, entries, rcs, starts) -> None:
+        """Real rows first, then pad rows that read and write the reserved pad page at position 0
+        (reference: engine/graphs.py:115-167)."""
+        pad = self.manager.get(PAD_REQUEST)
+        n_pad = g.size - len(entries)
+        slots = [rc.slot for rc in rcs] + [pad.slot] * n_pad
+        token_ids = [e.tokens[0] for e in entries] + [0] * n_pad
+        st = list(starts) + [0] * n_pad
+        tables = [t[slots, :] for t in self._tables]
+        fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables)
+        g.dev_buf.copy_(g.host, non_blocking=True)
+        self._staged = torch.cuda.Event()
+        self._staged.record(self.stream)
+
+    def _capture(self, size: int) -> _DecodeGraph:
+        g = _DecodeGraph(self, size)
+        self._fill_graph(g, [], [], [])
+        ctx = g.context(self)
+
+        def run():
+            g.arena.reset()
+            resid, delta = self.model.forward_hidden(ctx, self.storage.views)
+            return self.model.logits(ctx, resid, delta, ctx.want_rows)
+
+        run()  # warm-up: loads the libraries and lets the arena grow to what a step needs
+        self.stream.synchronize()
+        g.arena.reset()  # one chunk from here on
+        g.arena.fixed = True
+        graph = ops.Graph(self.stream)
+        with graph:
+            g.logits = run()
+        g.graph = graph
+        self._graphs[size] = g
+        return g
+
+    def _step_graph(self, entries, rcs, starts):
+        self._ensure_pad()
+        size = self._bucket(len(entries))
+        g = self._graphs.get(size) or self._capture(size)
+        max_kv = max(starts) + 1
+        if -(-max_kv // self.page_size) > self.table_width:
+            raise ValueError("a request is longer than the block tables of the captured graphs")
+        self._check_positions(max_kv - 1)
+        self._fill_graph(g, entries, rcs, starts)
+        g.graph.launch()
+        rows = [i for i, e in enumerate(entries) if e.want]
+        if len(rows) == len(entries):
+            return g.logits[: len(entries)]
+        return g.logits[rows]
+
+    def _check_positions(self, max_position: int) -> None:
+        for layer in self.model.layers:
+            limit = getattr(getattr(layer.mixer, "position", None), "max_positions", None)
+            if limit is not None and max_position >= limit:
+                raise ValueError(f"position {max_position} is beyond the model's {limit} positions")
+
+    def synchronize(self) -> None:
+        self.stream.synchronize()

@@ -1,0 +1,324 @@
+"""Python faces of the HIP kernels.  Each function checks on the host that the operands have the
+shapes, strides and types the kernel and its grid assume, then launches on the current stream.
+
+A size a kernel does not take raises ``KernelRefused`` with the reason; nothing is computed
+elsewhere instead.  Tensors are torch tensors on the GPU; only their addresses cross into C.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_size_t, c_uint32, c_void_p
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+
+
+class KernelRefused(Exception):
+    """A kernel was asked for a size or type it does not take."""
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise KernelRefused(f"kernels take float32 or bfloat16 tensors, not {t.dtype}")
+
+
+def _ptr(t):
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelRefused("kernels run on GPU tensors only; there is no CPU path")
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        lib = build.core()
+        lib.ns_error_string.restype = ctypes.c_char_p
+        msg = lib.ns_error_string(c_int(code)).decode()
+        raise KernelRefused(f"{what}: {msg} (code {code})")
+
+
+def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelRefused(f"{name} must be a contiguous int32 tensor")
+    return t
+
+
+# ------------------------------------------------------------------------------------------------ elementwise
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[i] = table[ids[i]].  ``ids`` int32; the caller has checked 0 <= id < vocab."""
+    _gpu(table, ids)
+    _i32(ids, "ids")
+    n, hidden = ids.numel(), table.shape[1]
+    if out is None:
+        out = torch.empty((n, hidden), dtype=table.dtype, device=table.device)
+    if not table.is_contiguous() or out.shape != (n, hidden) or out.dtype != table.dtype or not out.is_contiguous():
+        raise KernelRefused("embed: table and out must be contiguous [*, hidden] of one dtype")
+    _check(build.core().ns_embed(_ptr(out), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), c_int(_dtype_code(table)), _stream()), "embed")
+    return out
+
+
+def rmsnorm(weight: torch.Tensor, eps: float, resid: torch.Tensor | None = None, x: torch.Tensor | None = None,
+            rows: torch.Tensor | None = None, write_resid: bool = False, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[i] = weight * norm(resid[r] + x[r]) with r = rows[i] (or i).  With ``write_resid`` the sum
+    is also stored back into ``resid`` (not with ``rows``)."""
+    src = resid if resid is not None else x
+    if src is None:
+        raise KernelRefused("rmsnorm needs resid or x")
+    _gpu(weight, resid, x, rows)
+    dim = weight.numel()
+    for t in (resid, x):
+        if t is not None and (t.dim() != 2 or t.shape[1] != dim or not t.is_contiguous() or t.dtype != weight.dtype):
+            raise KernelRefused(f"rmsnorm: operands must be contiguous [*, {dim}] of the weight's dtype")
+    if resid is not None and x is not None and resid.shape != x.shape:
+        raise KernelRefused("rmsnorm: resid and x differ in shape")
+    if rows is not None:
+        _i32(rows, "rows")
+    n = rows.numel() if rows is not None else src.shape[0]
+    if out is None:
+        out = torch.empty((n, dim), dtype=weight.dtype, device=weight.device)
+    if out.shape != (n, dim) or not out.is_contiguous() or out.dtype != weight.dtype:
+        raise KernelRefused("rmsnorm: out has the wrong shape")
+    _check(build.core().ns_rmsnorm(_ptr(out), _ptr(resid), _ptr(x), _ptr(weight), _ptr(rows), c_int(n), c_int(dim), c_float(eps),
+                                   c_int(1 if write_resid else 0), c_int(_dtype_code(weight)), _stream()), "rmsnorm")
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor, block_table: torch.Tensor,
+                  inv_freq: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int, kv_heads: int,
+                  head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
+    """Rotate q in place inside ``qkv`` [N, (heads + 2 kv_heads) * head_dim]; rotate k and write k and v of
+    every token into the pages ``block_table[token_req[t], position // page]``.
+    k_cache [pages, page, kv_heads, head_dim]; v_cache [pages, kv_heads, head_dim, page]."""
+    _gpu(qkv, positions, token_req, block_table, inv_freq, k_cache, v_cache)
+    n = positions.numel()
+    width = (heads + 2 * kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[0] != n or qkv.shape[1] != width or qkv.stride(1) != 1:
+        raise KernelRefused(f"rope_kv_write: qkv must be [{n}, {width}]")
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
+    if token_req.numel() != n or block_table.dim() != 2:
+        raise KernelRefused("rope_kv_write: token_req is per token, block_table is [requests, pages]")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2:
+        raise KernelRefused("rope_kv_write: inv_freq must hold rotary_dim/2 float32 values")
+    page = k_cache.shape[1]
+    if (k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+            or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("rope_kv_write: cache pages do not fit heads, head size or dtype")
+    _check(build.core().ns_rope_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
+                                         c_int(block_table.stride(0)), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(n),
+                                         c_int(heads), c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(page),
+                                         c_int(1 if write_kv else 0), c_int(_dtype_code(qkv)), _stream()), "rope_kv_write")
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[n, i] = silu(gu[n, i]) * gu[n, I + i] for gu [N, 2 I]."""
+    _gpu(gu)
+    n, two_i = gu.shape
+    inter = two_i // 2
+    if two_i % 2 or not gu.is_contiguous():
+        raise KernelRefused("silu_mul: gu must be contiguous [N, 2 I]")
+    if out is None:
+        out = torch.empty((n, inter), dtype=gu.dtype, device=gu.device)
+    _check(build.core().ns_silu_mul(_ptr(out), _ptr(gu), c_int(n), c_int(inter), c_int(_dtype_code(gu)), _stream()), "silu_mul")
+    return out
+
+
+def fill_u32(t: torch.Tensor, value: int = 0) -> None:
+    """Set every 32-bit word of ``t`` (a kernel, so that it may be part of a captured graph)."""
+    _gpu(t)
+    nbytes = t.numel() * t.element_size()
+    if nbytes % 4 or not t.is_contiguous():
+        raise KernelRefused("fill_u32: the tensor must be contiguous and a whole number of 32-bit words")
+    _check(build.core().ns_fill_u32(_ptr(t), c_uint32(value), c_size_t(nbytes // 4), _stream()), "fill_u32")
+
+
+# ------------------------------------------------------------------------------------------------ matrix products
+
+
+def _check_linear(x, w, out, out_f32):
+    _gpu(x, w, out)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or not w.is_contiguous() or x.dtype != w.dtype:
+        raise KernelRefused(f"linear: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit (w is [out, in], one dtype)")
+    m, n = x.shape[0], w.shape[0]
+    want = torch.float32 if out_f32 else x.dtype
+    if out is None:
+        out = torch.empty((m, n), dtype=want, device=x.device)
+    if out.shape != (m, n) or out.dtype != want or out.stride(1) != 1:
+        raise KernelRefused("linear: out has the wrong shape or dtype")
+    return out
+
+
+def linear_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False) -> torch.Tensor:
+    """x @ w.T with the plain tiled kernel: any sizes, float32 or bfloat16, 32-bit accumulation in a fixed order."""
+    out = _check_linear(x, w, out, out_f32)
+    m, k = x.shape
+    _check(build.core().ns_gemm_generic(_ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(w.shape[0]), c_int(k), c_int(x.stride(0)),
+                                        c_int(out.stride(0)), c_int(1 if out_f32 else 0), c_int(_dtype_code(x)), _stream()), "linear_generic")
+    return out
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_takes(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and w.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def linear_skinny(x: torch.Tensor, w: torch.Tensor, w2: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                  out_f32: bool = False, waves: int = 0) -> torch.Tensor:
+    """bfloat16 x @ w.T for at most 64 rows on the matrix cores; with ``w2``: silu(x @ w.T) * (x @ w2.T)."""
+    out = _check_linear(x, w, out, out_f32)
+    if not skinny_takes(x, w):
+        raise KernelRefused(f"linear_skinny takes bfloat16, at most {SKINNY_MAX_ROWS} rows and an inner size that is a multiple of 8; "
+                            f"got x {tuple(x.shape)} {x.dtype}")
+    if w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous() or w2.data_ptr() % 16):
+        raise KernelRefused("linear_skinny: w2 must match w")
+    m, k = x.shape
+    if waves == 0:
+        # enough waves in flight to keep the memory system busy: 8 waves share K when a launch has few workgroups
+        waves = 8 if (w.shape[0] + 15) // 16 < 1024 and k >= 2048 else 4
+    _check(build.core().ns_gemm_skinny_bf16(_ptr(out), _ptr(x), _ptr(w), _ptr(w2), c_int(m), c_int(w.shape[0]), c_int(k),
+                                            c_int(x.stride(0)), c_int(out.stride(0)), c_int(1 if w2 is not None else 0),
+                                            c_int(1 if out_f32 else 0), c_int(waves), _stream()), "linear_skinny")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ attention
+
+
+def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim):
+    _gpu(q, out, k_cache, v_cache)
+    page = k_cache.shape[1]
+    if (k_cache.dim() != 4 or k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+            or not k_cache.is_contiguous() or not v_cache.is_contiguous() or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype):
+        raise KernelRefused("attention: cache pages do not fit heads, head size or dtype")
+    if q.stride(1) != 1 or q.shape[1] < heads * head_dim:
+        raise KernelRefused("attention: q rows must hold heads * head_dim contiguous values")
+    if out.shape != (q.shape[0], heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelRefused("attention: out must be contiguous [tokens, heads * head_dim]")
+    if heads % kv_heads:
+        raise KernelRefused(f"attention: {heads} heads are not a multiple of {kv_heads} key/value heads")
+    return page
+
+
+def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_table, heads: int, kv_heads: int, head_dim: int,
+                      scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of every token's query over its request's pages; any head size up to 256, either dtype."""
+    page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
+    _i32(token_req, "token_req"), _i32(positions, "positions"), _i32(block_table, "block_table")
+    if head_dim > 256:
+        raise KernelRefused(f"attention_generic takes head sizes up to 256, not {head_dim}")
+    n = q.shape[0]
+    _check(build.core().ns_attn_generic(_ptr(out), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(token_req),
+                                        _ptr(positions), _ptr(block_table), c_int(block_table.stride(0)), c_int(n), c_int(heads),
+                                        c_int(kv_heads), c_int(head_dim), c_int(page), c_float(scale), c_int(window),
+                                        c_int(_dtype_code(q)), _stream()), "attention_generic")
+    return out
+
+
+def mfma_attention_takes(dtype, head_dim: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and page_size % 4 == 0
+
+
+def attention_mfma(q, out, k_cache, v_cache, tile_req, tile_t0, qo_indptr, kv_lens, block_table, heads: int, kv_heads: int,
+                   head_dim: int, scale: float, window: int = 0, hp: int = 1, splits: int = 1,
+                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+    """bfloat16 attention on the matrix cores for the tiles (request, first token) listed in ``tile_req`` /
+    ``tile_t0``.  ``hp`` heads of a group times 16/hp tokens make a tile; ``splits`` > 1 cuts the keys of
+    every tile into that many ranges and needs ``workspace`` = (part_o, part_ml) float32 tensors."""
+    page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
+    if not mfma_attention_takes(q.dtype, head_dim, page):
+        raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
+                            f"multiples of 4; got {q.dtype}, head size {head_dim}, page {page}")
+    for name, t in (("tile_req", tile_req), ("tile_t0", tile_t0), ("qo_indptr", qo_indptr), ("kv_lens", kv_lens), ("block_table", block_table)):
+        _gpu(t)
+        _i32(t, name)
+    n_tiles, n_tokens = tile_req.numel(), q.shape[0]
+    po = pm = None
+    if splits > 1:
+        if workspace is None:
+            raise KernelRefused("attention_mfma: splits > 1 needs a workspace")
+        po, pm = workspace
+        if po.dtype != torch.float32 or pm.dtype != torch.float32 or po.numel() < n_tokens * heads * splits * head_dim or pm.numel() < n_tokens * heads * splits * 2:
+            raise KernelRefused("attention_mfma: workspace too small")
+    lib = build.attn(head_dim)
+    _check(lib.ns_attn_mfma(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tile_req),
+                            _ptr(tile_t0), _ptr(qo_indptr), _ptr(kv_lens), _ptr(block_table), c_int(block_table.stride(0)),
+                            c_int(n_tiles), c_int(n_tokens), c_int(heads), c_int(kv_heads), c_int(page), c_int(hp), c_int(splits),
+                            c_int(window), c_float(scale), _stream()), "attention_mfma")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ sampling
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, top_k: torch.Tensor | None = None,
+           top_p: torch.Tensor | None = None):
+    """Per row of float32 ``logits``: arg-max when temperature is 0, else a draw by inverse CDF with the
+    row's uniform number.  -> (token int32, log-probability of it under the raw logits, log-probability
+    under the processed distribution; 0 for arg-max rows)."""
+    _gpu(logits, temperature, uniform, top_k, top_p)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelRefused("sample: logits must be float32 [rows, vocab]")
+    rows, vocab = logits.shape
+    for name, t, dt in (("temperature", temperature, torch.float32), ("uniform", uniform, torch.float32),
+                        ("top_k", top_k, torch.int32), ("top_p", top_p, torch.float32)):
+        if t is not None and (t.dtype != dt or t.numel() != rows or not t.is_contiguous()):
+            raise KernelRefused(f"sample: {name} must hold one {dt} per row")
+    tok = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    lp = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    slp = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    _check(build.core().ns_sample(_ptr(tok), _ptr(lp), _ptr(slp), _ptr(logits), c_int(logits.stride(0)), _ptr(temperature),
+                                  _ptr(top_k), _ptr(top_p), _ptr(uniform), c_int(rows), c_int(vocab), _stream()), "sample")
+    return tok, lp, slp
+
+
+# ------------------------------------------------------------------------------------------------ graphs
+
+
+class Graph:
+    """A captured stream of launches.  ``with Graph.capture(stream) as g: ...`` then ``g.launch()``."""
+
+    def __init__(self, stream: torch.cuda.Stream) -> None:
+        self.stream, self._exec = stream, None
+
+    def __enter__(self):
+        self._ctx = torch.cuda.stream(self.stream)
+        self._ctx.__enter__()
+        _check(build.core().ns_graph_begin(c_void_p(self.stream.cuda_stream)), "graph capture begin")
+        return self
+
+    def __exit__(self, et, ev, tb):
+        handle = c_void_p()
+        code = build.core().ns_graph_end(c_void_p(self.stream.cuda_stream), ctypes.byref(handle))
+        self._ctx.__exit__(et, ev, tb)
+        if et is None:
+            _check(code, "graph capture end")
+            self._exec = handle
+        return False
+
+    def launch(self) -> None:
+        _check(build.core().ns_graph_launch(self._exec, c_void_p(self.stream.cuda_stream)), "graph launch")
+
+    def __del__(self):
+        if getattr(self, "_exec", None):
+            try:
+                build.core().ns_graph_destroy(self._exec)
+            except Exception:
+                pass

@@ -1,0 +1,90 @@
+"""Grouped-query soft-max attention over the paged cache (reference: model/llama.py:161-184 and
+model/attention.py).
+
+Per step: one product for q, k and v together (the three checkpoint matrices are stacked at load
+time), rotation of q and k fused with the write of k and v into the pages, attention of every token
+over its request's pages, output projection.  float32 runs the plain attention kernel; bfloat16 runs
+the matrix-core kernel: prompt portions as tiles of 16 tokens of one head, decode rows as tiles of
+all heads of a group with the keys cut into ranges that are joined afterwards.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from . import registry
+from .linear import linear
+from .needs import PagedNeed
+
+
+class Attention:
+    graph_safe = True
+
+    def __init__(self, spec, prefix: str) -> None:
+        if spec.heads % spec.kv_heads:
+            raise ValueError(f"{spec.heads} heads are not a multiple of {spec.kv_heads} key/value heads")
+        self.spec, self.prefix = spec, prefix
+        self.position = registry.build("position", spec.position, prefix)
+        if self.position.rotary_dim > spec.head_dim:
+            raise ValueError("the rotary part of a head cannot be wider than the head")
+        self.wqkv: torch.Tensor | None = None
+        self.wo: torch.Tensor | None = None
+
+    @property
+    def _names(self):
+        p = self.prefix
+        return p + "q_proj.weight", p + "k_proj.weight", p + "v_proj.weight", p + "o_proj.weight"
+
+    def wanted(self) -> dict:
+        s = self.spec
+        q, k, v, o = self._names
+        return {
+            q: ((s.heads * s.head_dim, s.hidden), "linear"),
+            k: ((s.kv_heads * s.head_dim, s.hidden), "linear"),
+            v: ((s.kv_heads * s.head_dim, s.hidden), "linear"),
+            o: ((s.hidden, s.heads * s.head_dim), "linear"),
+            **self.position.wanted(),
+        }
+
+    def load(self, get, dtype, device) -> None:
+        s = self.spec
+        q, k, v, o = self._names
+        rows = (s.heads + 2 * s.kv_heads) * s.head_dim
+        self.wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
+        at = 0
+        for name in (q, k, v):
+            t = get(name)
+            self.wqkv[at : at + t.shape[0]].copy_(t)
+            at += t.shape[0]
+        self.wo = get(o).to(device=device, dtype=dtype).contiguous()
+        self.position.load(get, dtype, device)
+
+    def cache_need(self):
+        return PagedNeed(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
+
+    def forward(self, ctx, x: torch.Tensor, cache, owns_cache: bool = True, out: torch.Tensor | None = None) -> torch.Tensor:
+        s = self.spec
+        n = x.shape[0]
+        pos = self.position
+        if pos.max_positions is not None and ctx.max_position >= pos.max_positions:
+            raise ValueError(f"position {ctx.max_position} is beyond the model's {pos.max_positions} positions")
+        qkv = linear(x, self.wqkv, out=ctx.arena.take(((n, self.wqkv.shape[0])), x.dtype))
+        table = ctx.block_tables[cache.group]
+        ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
+                          s.head_dim, pos.rotary_dim, write_kv=owns_cache)
+        att = ctx.arena.take((n, s.heads * s.head_dim), x.dtype)
+        page = cache.k.shape[1]
+        if ops.mfma_attention_takes(x.dtype, s.head_dim, page):
+            group = s.heads // s.kv_heads
+            for plan in ctx.attention_plans(group, s.kv_heads, s.head_dim):
+                ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tile_req, plan.tile_t0, ctx.qo_indptr, ctx.kv_lens, table,
+                                   s.heads, s.kv_heads, s.head_dim, s.softmax_scale, window=s.window, hp=plan.hp,
+                                   splits=plan.splits, workspace=plan.workspace)
+        else:
+            ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
+                                  s.head_dim, s.softmax_scale, window=s.window)
+        return linear(att, self.wo, out=out)
+
+
+registry.register("mixer", "attention", Attention)

@@ -1,0 +1,88 @@
+"""A model built from a ``ModelSpec``: embedding, the layers in their run order, the last norm and
+the output head (reference: model/llama.py:211-286).  Nothing here knows an architecture's name."""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights import source as wsource
+from . import registry
+from .linear import linear
+from .needs import PagedNeed, StateNeed
+
+
+def _build_layers(spec):
+    return [registry.build("block", layer, None) for layer in spec.layers]
+
+
+def wanted_tensors(spec, layers=None) -> dict:
+    """Every tensor the model reads from a checkpoint: name -> (shape, role)."""
+    layers = layers if layers is not None else _build_layers(spec)
+    out = {spec.embed_name: ((spec.vocab_size, spec.hidden), "embedding")}
+    for layer in layers:
+        out.update(layer.wanted())
+    out.update(registry.build("norm", spec.final_norm, spec.final_norm_name).wanted())
+    out[spec.head_name] = ((spec.vocab_size, spec.hidden), "linear")
+    return out
+
+
+class DecoderModel:
+    def __init__(self, spec, config=None) -> None:
+        self.spec, self.config = spec, config
+        self.layers = _build_layers(spec)
+        self.final_norm = registry.build("norm", spec.final_norm, spec.final_norm_name)
+        self.embed: torch.Tensor | None = None
+        self.head: torch.Tensor | None = None
+        self.dtype = self.device = None
+        # what every entry of the run order keeps in the cache
+        self.cache_needs = [self.layers[c.layer].cache_need() if c.cache_from is None else None for c in spec.run_order]
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(layer.graph_safe for layer in self.layers)
+
+    def wanted(self) -> dict:
+        return wanted_tensors(self.spec, self.layers)
+
+    def load(self, source, dtype: torch.dtype, device) -> "DecoderModel":
+        """Check the source against what the model wants (one error that lists everything wrong), then read
+        each tensor once.  A head that is absent is the embedding table if the configuration ties them
+        (reference: model/loader.py:62-70)."""
+        spec = self.spec
+        wanted = {k: v[0] for k, v in self.wanted().items()}
+        wsource.check(source, wanted, optional={spec.head_name} if spec.tie_head else frozenset())
+        self.dtype, self.device = dtype, torch.device(device)
+        get = source.get
+        self.embed = get(spec.embed_name).to(device=device, dtype=dtype).contiguous()
+        if spec.head_name in source.names():
+            self.head = get(spec.head_name).to(device=device, dtype=dtype).contiguous()
+        else:
+            self.head = self.embed  # one storage
+        for layer in self.layers:
+            layer.load(get, dtype, device)
+        self.final_norm.load(get, dtype, device)
+        return self
+
+    # ------------------------------------------------------------------ one pass over the given tokens
+
+    def forward_hidden(self, ctx, caches) -> tuple[torch.Tensor, torch.Tensor]:
+        """Run the tokens of ``ctx`` through every entry of the run order.  -> (resid, delta): the stream
+        before the last sum.  ``caches[i]`` is the cache view of run-order entry i (its own or the one
+        it reads)."""
+        n = ctx.n_tokens
+        resid = ctx.arena.take((n, self.spec.hidden), self.dtype)
+        delta = ctx.arena.take((n, self.spec.hidden), self.dtype)
+        ops.embed(self.embed, ctx.token_ids, out=resid)
+        pending = None
+        for i, call in enumerate(self.spec.run_order):
+            self.layers[call.layer].forward(ctx, resid, pending, caches[i], call.cache_from is None, delta)
+            pending = delta
+        return resid, pending
+
+    def logits(self, ctx, resid, delta, rows: torch.Tensor) -> torch.Tensor:
+        """32-bit logits [len(rows), vocab] at the given token rows: last sum, last norm and head only there
+        (reference: model/llama.py:284-286, engine/engine.py:382)."""
+        n = rows.numel()
+        h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
+        return linear(h, self.head, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True)

@@ -1,0 +1,47 @@
+"""Which class implements which kind of part.
+
+A role ("norm", "position", "mixer", "ffn", "block") and a spec's ``kind`` name a class.  A new part is
+registered once with ``register(role, kind, cls)``, from anywhere (a test registers toy parts), and is
+then built wherever a spec of that kind appears in a ``ModelSpec``.
+
+What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are [tokens, width]):
+
+  every part   __init__(spec, prefix)             prefix: tensor-name prefix of its weights
+               wanted() -> {name: (shape, role)}   tensors it reads from the checkpoint; role is one of
+                                                  "linear" | "embedding" | "norm" (used by random init)
+               load(get, dtype, device)           get(name) returns the stored tensor (CPU)
+               graph_safe: bool                   True if forward only launches kernels on the current
+                                                  stream into buffers taken from ctx.arena
+  norm         forward(ctx, resid=None, x=None, rows=None, write_resid=False, out=None)
+                                                  normalise resid + x (the sum optionally stored back)
+  position     an object the mixer that owns it knows how to use (rope: ``inv_freq`` on the device)
+  mixer        cache_need() -> PagedNeed | StateNeed | None
+               forward(ctx, x, cache, owns_cache, out=None) -> [tokens, hidden]
+  ffn          forward(ctx, x, out=None) -> [tokens, hidden]
+  block        forward(ctx, resid, delta, cache, owns_cache, delta_out) -> None
+                                                  resid is updated in place; the not yet added output of
+                                                  the block's last part is left in delta_out
+"""
+
+from __future__ import annotations
+
+_PARTS: dict[tuple[str, str], type] = {}
+ROLES = ("norm", "position", "mixer", "ffn", "block")
+
+
+def register(role: str, kind: str, cls: type) -> None:
+    if role not in ROLES:
+        raise ValueError(f"unknown role {role!r}; roles are {ROLES}")
+    _PARTS[(role, kind)] = cls
+
+
+def build(role: str, spec, prefix: str):
+    kind = getattr(spec, "kind", None)
+    if (role, kind) not in _PARTS:
+        known = sorted(k for r, k in _PARTS if r == role)
+        raise ValueError(f"no {role} of kind {kind!r} is registered (known: {known})")
+    return _PARTS[(role, kind)](spec, prefix)
+
+
+def registered(role: str) -> list[str]:
+    return sorted(k for r, k in _PARTS if r == role)

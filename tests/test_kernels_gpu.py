@@ -1,0 +1,384 @@
+"""Each kernel alone against its plain reference, at sizes other than the engine tests use."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+import plain_llama as pl
+from tiny import ulps_of_row_max
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _ops():
+    from nanospec_amd.kernels import ops
+
+    return ops
+
+
+def _tol(dtype):
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    ops = _ops()
+    table = torch.randn(301, 72, dtype=dtype, device=DEV)
+    ids = torch.tensor([0, 300, 5, 5, 17], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.embed(table, ids), table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dim", [72, 1000, 4096])
+def test_rmsnorm_plain_fused_and_gathered(dtype, dim):
+    ops = _ops()
+    torch.manual_seed(dim)
+    n, eps = 7, 3e-6
+    resid = torch.randn(n, dim, dtype=dtype, device=DEV) * 3
+    x = torch.randn(n, dim, dtype=dtype, device=DEV)
+    w = (1 + 0.1 * torch.randn(dim, device=DEV)).to(dtype)
+    # plain
+    ref = pl.rms_norm(resid.cpu(), w.cpu(), eps)
+    torch.testing.assert_close(ops.rmsnorm(w, eps, resid=resid).cpu(), ref, **_tol(dtype))
+    # fused sum, written back
+    r2 = resid.clone()
+    out = ops.rmsnorm(w, eps, resid=r2, x=x, write_resid=True)
+    summed = pl.residual_add(resid.cpu(), x.cpu())
+    assert torch.equal(r2.cpu(), summed)
+    torch.testing.assert_close(out.cpu(), pl.rms_norm(summed, w.cpu(), eps), **_tol(dtype))
+    # gathered rows, nothing written
+    rows = torch.tensor([6, 0, 6, 3], dtype=torch.int32, device=DEV)
+    r3 = resid.clone()
+    out = ops.rmsnorm(w, eps, resid=r3, x=x, rows=rows)
+    assert torch.equal(r3, resid)
+    torch.testing.assert_close(out.cpu(), pl.rms_norm(summed, w.cpu(), eps)[rows.cpu().long()], **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1, 40, 24), (5, 130, 200), (70, 65, 17), (200, 300, 128)])
+def test_linear_generic(dtype, m, n, k):
+    ops = _ops()
+    torch.manual_seed(m * n)
+    x = torch.randn(m, k, dtype=dtype, device=DEV)
+    w = torch.randn(n, k, dtype=dtype, device=DEV)
+    ref = x.cpu().float() @ w.cpu().float().T
+    out = ops.linear_generic(x, w, out_f32=True)
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-4)
+    out2 = ops.linear_generic(x, w)
+    torch.testing.assert_close(out2.cpu().float(), ref.to(dtype).float(), **_tol(dtype))
+    # a row's result does not depend on the rows beside it
+    assert torch.equal(ops.linear_generic(x[:1].contiguous(), w, out_f32=True), out[:1])
+
+
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064)])
+def test_linear_skinny(m, n, k):
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m, k, dtype=torch.bfloat16, device=DEV)
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    ref = x.cpu().float() @ w.cpu().float().T
+    for waves in (4, 8):
+        out = ops.linear_skinny(x, w, out_f32=True, waves=waves)
+        torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
+    out = ops.linear_skinny(x, w)
+    assert ulps_of_row_max(out.cpu(), ref).max() <= 1.0
+    # fused silu(gate) * up
+    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    g, u = ref, x.cpu().float() @ w2.cpu().float().T
+    act = ops.linear_skinny(x, w, w2=w2)
+    want = g * torch.sigmoid(g) * u
+    assert ulps_of_row_max(act.cpu(), want).max() <= 1.0
+
+
+def test_linear_skinny_refuses():
+    ops = _ops()
+    from nanospec_amd.kernels import KernelRefused
+
+    x = torch.randn(65, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.randn(16, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelRefused):
+        ops.linear_skinny(x, w)
+    with pytest.raises(KernelRefused):
+        ops.linear_skinny(x[:4, :60], w[:, :60].contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul(dtype):
+    ops = _ops()
+    gu = torch.randn(9, 2 * 88, dtype=dtype, device=DEV) * 3
+    g, u = gu.cpu().float()[:, :88], gu.cpu().float()[:, 88:]
+    torch.testing.assert_close(ops.silu_mul(gu).cpu().float(), (torch.nn.functional.silu(g) * u).to(dtype).float(), **_tol(dtype))
+
+
+# ------------------------------------------------------------------------------------------------ cache helpers
+
+
+def make_cache(pages, page, kvh, hd, dtype):
+    k = torch.zeros(pages, page, kvh, hd, dtype=dtype, device=DEV)
+    v = torch.zeros(pages, kvh, hd, page, dtype=dtype, device=DEV)
+    return k, v
+
+
+def scattered_tables(lens, page, pages, seed=0):
+    """Block tables on scattered, non-contiguous pages."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(pages, generator=g).tolist()
+    width = max(-(-n // page) for n in lens)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    for b, n in enumerate(lens):
+        for i in range(-(-n // page)):
+            table[b, i] = perm.pop()
+    return table
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rot", [24, 16, 0])
+def test_rope_kv_write(dtype, rot):
+    """q rotated in place, k rotated into its page slot, v into the transposed page; against the plain rotation."""
+    ops = _ops()
+    torch.manual_seed(1)
+    heads, kvh, hd, page = 6, 3, 24, 4
+    starts, lens = [0, 5, 9], [7, 1, 3]
+    n = sum(lens)
+    table = scattered_tables([s + l for s, l in zip(starts, lens)], page, 16).to(DEV)
+    positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    qkv = torch.randn(n, (heads + 2 * kvh) * hd, dtype=dtype, device=DEV)
+    before = qkv.clone().cpu()
+    k, v = make_cache(16, page, kvh, hd, dtype)
+    inv = pl.inverse_frequencies(rot, 10000.0, None) if rot else torch.zeros(1)
+    ops.rope_kv_write(qkv, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot)
+    q0 = before[:, : heads * hd].view(n, heads, hd)
+    k0 = before[:, heads * hd : (heads + kvh) * hd].view(n, kvh, hd)
+    v0 = before[:, (heads + kvh) * hd :].view(n, kvh, hd)
+    if rot:
+        cos, sin = pl.rotation_tables(positions.cpu(), inv)
+        q_ref = torch.cat([pl.rotate(q0[..., :rot], cos, sin), q0[..., rot:]], -1)
+        k_ref = torch.cat([pl.rotate(k0[..., :rot], cos, sin), k0[..., rot:]], -1)
+    else:
+        q_ref, k_ref = q0, k0
+    tol = _tol(dtype)
+    torch.testing.assert_close(qkv.cpu()[:, : heads * hd].view(n, heads, hd).float(), q_ref.float(), **tol)
+    assert torch.equal(qkv.cpu()[:, heads * hd :], before[:, heads * hd :])  # k and v stay as they were in the buffer
+    for t in range(n):
+        b, p = int(token_req[t]), int(positions[t])
+        pg, off = int(table[b, p // page]), p % page
+        torch.testing.assert_close(k[pg, off].cpu().float(), k_ref[t].float(), **tol)
+        assert torch.equal(v[pg, :, :, off].cpu(), v0[t])
+
+
+def fill_cache(k, v, table, lens, page, kvh, hd, dtype, seed=0, scale=1.0):
+    """Random keys and values for positions [0, len) of every request, written through the block table.
+    -> per request (K [len, kvh, hd], V [len, kvh, hd]) on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for b, n in enumerate(lens):
+        kk = (torch.randn(n, kvh, hd, generator=g) * scale).to(dtype)
+        vv = torch.randn(n, kvh, hd, generator=g).to(dtype)
+        for p in range(n):
+            pg, off = int(table[b, p // page]), p % page
+            if pg < 0:
+                continue
+            k[pg, off] = kk[p].to(DEV)
+            v[pg, :, :, off] = vv[p].to(DEV)
+        out.append((kk, vv))
+    return out
+
+
+def plain_paged_attention(q, kvs, starts, lens, heads, scale_fix=1.0, window=0):
+    """Rows of q (flat over requests) attend to their request's keys 0 .. position with the plain attention."""
+    outs, at = [], 0
+    for (kk, vv), s, n in zip(kvs, starts, lens):
+        qi = q[at : at + n]
+        o = pl.causal_attention(qi.cpu(), kk[: s + n], vv[: s + n], first_query=s)
+        if window:
+            o = torch.stack([pl.causal_attention(qi[i : i + 1].cpu(), kk[max(0, s + i - window + 1) : s + i + 1],
+                                                 vv[max(0, s + i - window + 1) : s + i + 1], first_query=min(s + i, window - 1))[0]
+                             for i in range(n)])
+        outs.append(o)
+        at += n
+    return torch.cat(outs)
+
+
+CASES = {
+    # the four cases of the reference's tests/test_backends.py:44-59
+    "prefill": ([0], [40]),
+    "decode": ([37], [1]),
+    "append6": ([37], [6]),
+    "mixed": ([21, 50, 0], [1, 6, 9]),
+    "long": ([300, 0, 511], [1, 70, 1]),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", list(CASES))
+@pytest.mark.parametrize("heads,kvh,hd,page", [(8, 2, 128, 16), (6, 1, 48, 4), (4, 4, 16, 8)])
+def test_attention_generic(dtype, case, heads, kvh, hd, page):
+    ops = _ops()
+    starts, lens = CASES[case]
+    torch.manual_seed(3)
+    total = [s + l for s, l in zip(starts, lens)]
+    pages = sum(-(-t // page) for t in total) + 3
+    table = scattered_tables(total, page, pages)
+    k, v = make_cache(pages, page, kvh, hd, dtype)
+    kvs = fill_cache(k, v, table, total, page, kvh, hd, dtype)
+    n = sum(lens)
+    q = torch.randn(n, heads * hd, dtype=dtype, device=DEV)
+    positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    out = torch.empty(n, heads * hd, dtype=dtype, device=DEV)
+    ops.attention_generic(q, out, k, v, token_req, positions, table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd))
+    ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
+    if dtype == torch.float32:
+        torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-5)
+    else:
+        assert ulps_of_row_max(out.cpu(), ref).max() <= 4  # the reference's bound, tests/test_backends.py:71
+
+
+def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None):
+    n = sum(lens)
+    B = len(lens)
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    kv_lens = torch.tensor([s + l for s, l in zip(starts, lens)], dtype=torch.int32, device=DEV)
+    out = torch.zeros(n, heads * hd, dtype=torch.bfloat16, device=DEV)
+    group = heads // kvh
+    ct = [(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16)]
+    dt = [(b, 0) for b, l in enumerate(lens) if l == 1]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    if ct:
+        ops.attention_mfma(q, out, k, v, i32([c[0] for c in ct]), i32([c[1] for c in ct]), indptr, kv_lens, table.to(DEV), heads, kvh,
+                           hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1)
+    if dt:
+        hp = 1
+        while hp < min(group, 16):
+            hp *= 2
+        splits = force_splits or 3
+        ws = (torch.empty(n * heads * splits * hd, dtype=torch.float32, device=DEV), torch.empty(n * heads * splits * 2, dtype=torch.float32, device=DEV))
+        ops.attention_mfma(q, out, k, v, i32([d[0] for d in dt]), i32([0] * len(dt)), indptr, kv_lens, table.to(DEV), heads, kvh, hd,
+                           1 / math.sqrt(hd), window=window, hp=hp, splits=splits, workspace=ws if splits > 1 else None)
+    return out
+
+
+@pytest.mark.parametrize("case", list(CASES))
+@pytest.mark.parametrize("heads,kvh,hd,page", [(8, 2, 128, 16), (6, 1, 48, 4), (4, 4, 16, 8), (32, 8, 64, 16), (40, 2, 32, 16)])
+def test_attention_mfma(case, heads, kvh, hd, page):
+    ops = _ops()
+    starts, lens = CASES[case]
+    torch.manual_seed(4)
+    total = [s + l for s, l in zip(starts, lens)]
+    pages = sum(-(-t // page) for t in total) + 3
+    table = scattered_tables(total, page, pages, seed=1)
+    k, v = make_cache(pages, page, kvh, hd, torch.bfloat16)
+    kvs = fill_cache(k, v, table, total, page, kvh, hd, torch.bfloat16, seed=2)
+    n = sum(lens)
+    q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
+    ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
+    for splits in (1, 3, 7):
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits)
+        u = ulps_of_row_max(out.cpu(), ref).max()
+        assert u <= 4, f"{case} splits={splits}: {u:.2f} ulps"
+
+
+@pytest.mark.parametrize("kernel", ["generic", "mfma"])
+def test_attention_far_key_and_page_edges(kernel):
+    """One key among hundreds is made to dominate: its score stands out, so the output must be its value.
+    Done for a key at every offset around page edges, so that a wrong page or slot shows."""
+    ops = _ops()
+    heads, kvh, hd, page = 4, 2, 32, 8
+    total, dtype = 333, torch.bfloat16
+    pages = -(-total // page) + 2
+    table = scattered_tables([total], page, pages, seed=5)
+    for special in (0, 7, 8, 9, 15, 16, 255, 256, 320, 331, 332):
+        k, v = make_cache(pages, page, kvh, hd, dtype)
+        kvs = fill_cache(k, v, table, [total], page, kvh, hd, dtype, seed=special, scale=0.05)
+        q = torch.randn(1, heads * hd, dtype=dtype, device=DEV)
+        pg, off = int(table[0, special // page]), special % page
+        for h in range(kvh):
+            k[pg, off, h] = (q.view(heads, hd)[h * (heads // kvh)] * 4).to(dtype)  # aligned with the group's first query head
+        starts, lens = [total - 1], [1]
+        if kernel == "mfma":
+            out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd)
+        else:
+            out = torch.empty_like(q)
+            ops.attention_generic(q, out, k, v, torch.zeros(1, dtype=torch.int32, device=DEV),
+                                  torch.tensor([total - 1], dtype=torch.int32, device=DEV), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd))
+        for h in range(kvh):
+            got = out.view(heads, hd)[h * (heads // kvh)].float().cpu()
+            want = kvs[0][1][special, h].float()
+            assert torch.allclose(got, want, atol=0.05), f"key {special}: output is not its value"
+
+
+@pytest.mark.parametrize("kernel", ["generic", "mfma"])
+@pytest.mark.parametrize("window", [5, 16, 40])
+def test_attention_window(kernel, window):
+    ops = _ops()
+    heads, kvh, hd, page = 4, 2, 32, 8
+    starts, lens = [50, 0, 100], [1, 45, 20]
+    dtype = torch.bfloat16
+    total = [s + l for s, l in zip(starts, lens)]
+    pages = sum(-(-t // page) for t in total) + 2
+    table = scattered_tables(total, page, pages, seed=7)
+    k, v = make_cache(pages, page, kvh, hd, dtype)
+    kvs = fill_cache(k, v, table, total, page, kvh, hd, dtype, seed=8)
+    # pages wholly before every query's window are released: the kernel must not touch them
+    for b, (s, l) in enumerate(zip(starts, lens)):
+        first_needed = max(0, s - window + 1) // page
+        table[b, :first_needed] = -1
+    n = sum(lens)
+    q = torch.randn(n, heads * hd, dtype=dtype, device=DEV)
+    ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads, window=window).reshape(n, -1)
+    if kernel == "mfma":
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=window)
+    else:
+        positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+        token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+        out = torch.empty(n, heads * hd, dtype=dtype, device=DEV)
+        ops.attention_generic(q, out, k, v, token_req, positions, table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window)
+    assert ulps_of_row_max(out.cpu(), ref).max() <= 4
+
+
+def test_sample_greedy_and_temperature():
+    ops = _ops()
+    torch.manual_seed(0)
+    rows, vocab = 6, 1003
+    z = torch.randn(rows, vocab, device=DEV) * 3
+    z[2, 100] = z[2, 900] = z[2].max() + 1  # a tie: the lowest index wins
+    T = torch.tensor([0.0, 0.8, 0.0, 1.0, 0.7, 1.3], device=DEV)
+    u = torch.tensor([0.3, 0.9, 0.5, 0.0, 0.5, 0.9999], device=DEV)
+    tok, lp, slp = ops.sample(z, T, u)
+    zc = z.cpu()
+    for r in range(rows):
+        t = float(T[r])
+        if t == 0:
+            assert int(tok[r]) == int(zc[r].argmax()) or r == 2
+            assert float(slp[r]) == 0.0
+        else:
+            ref = pl.draw_token(pl.processed_logprobs(zc[r], t, 0, 1.0), float(u[r]))
+            assert abs(int(tok[r]) - ref) <= 1, (r, int(tok[r]), ref)  # the cumulative sums round differently
+            assert abs(float(slp[r]) - float(pl.processed_logprobs(zc[r], t, 0, 1.0)[int(tok[r])])) < 1e-4
+        assert abs(float(lp[r]) - float(torch.log_softmax(zc[r], -1)[int(tok[r])])) < 1e-4
+    assert int(tok[2]) == 100
+
+
+def test_sample_top_k_top_p():
+    ops = _ops()
+    torch.manual_seed(1)
+    vocab = 500
+    z = torch.randn(4, vocab, device=DEV) * 2
+    T = torch.tensor([0.7, 1.0, 1.0, 0.9], device=DEV)
+    k = torch.tensor([5, 0, 3, 0], dtype=torch.int32, device=DEV)
+    p = torch.tensor([1.0, 0.8, 0.5, 0.2], device=DEV)
+    for uu in (0.01, 0.37, 0.62, 0.999):
+        u = torch.full((4,), uu, device=DEV)
+        tok, lp, slp = ops.sample(z, T, u, top_k=k, top_p=p)
+        for r in range(4):
+            ref_lp = pl.processed_logprobs(z[r].cpu(), float(T[r]), int(k[r]), float(p[r]))
+            ref = pl.draw_token(ref_lp, uu)
+            assert ref_lp[int(tok[r])] > -math.inf, "a token outside the kept set was drawn"
+            assert int(tok[r]) == ref, (r, uu, int(tok[r]), ref)
+            assert abs(float(slp[r]) - float(ref_lp[ref])) < 1e-4

@@ -1,0 +1,137 @@
+"""The engine's step function against the plain implementation, in 32-bit and in bfloat16, for the same requests
+cut into steps in four ways.  The logits at a position must not depend on the cut, the batch or the pages."""
+
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+import plain_llama as pl
+import traces
+from tiny import TINY, random_tokens, ulps_of_row_max
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+LENGTHS = {"A": (5, 17, 33, 64, 97, 128), "B": (1, 9, 40, 100, 130, 255)}
+
+
+def sequences(name):
+    vocab = TINY[name]["cfg"]["vocab_size"]
+    return {f"r{i}": random_tokens(n, vocab, 100 * i + n) for i, n in enumerate(LENGTHS[name])}
+
+
+_PLAIN = {}
+
+
+def plain_logits(folder, name, dtype):
+    key = (name, dtype)
+    if key not in _PLAIN:
+        cfg, w = pl.read_config(folder), pl.read_weights(folder, dtype)
+        _PLAIN[key] = {rid: pl.logits_of_sequence(w, cfg, toks, dtype) for rid, toks in sequences(name).items()}
+    return _PLAIN[key]
+
+
+_MODELS = {}
+
+
+def engine_model(folder, name, dtype):
+    from nanospec_amd.loader import load_model
+
+    key = (name, dtype)
+    if key not in _MODELS:
+        _MODELS[key] = load_model(folder, dtype=dtype)
+    return _MODELS[key]
+
+
+def check(ours: torch.Tensor, ref: torch.Tensor, dtype, what: str):
+    assert ours.shape == ref.shape, (what, ours.shape, ref.shape)
+    assert torch.isfinite(ours).all(), what
+    if dtype == torch.float32:
+        err = ((ours - ref).abs().amax(-1) / ref.abs().amax(-1)).max().item()
+        assert err <= 1e-4, f"{what}: {err:.2e} of the row's largest logit"
+    else:
+        u = ulps_of_row_max(ours, ref)
+        assert u.max() <= 8, f"{what}: {u.max():.2f} bf16 ulps of the row's largest logit (median {u.median():.2f})"
+
+
+def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True):
+    from nanospec_amd.engine.replay import Replayer
+
+    rep = Replayer(model, max_tokens, page_size=page, use_graphs=graphs)
+    for step, w in zip(steps, where):
+        out = rep.step(step["entries"], step["end"])
+        if not w:
+            assert out is None
+            continue
+        want = torch.stack([ref[rid][p] for rid, p in w])
+        check(out, want, dtype, f"step {step['step']} {[(e['id'], len(e['tokens'])) for e in step['entries']]}")
+    rep.manager.check()
+    live = [r for r in rep.manager.live if r != "__pad__"]
+    assert not live
+    return rep
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+def test_schedules_match_plain(tiny_folders, name, dtype, schedule):
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, dtype)
+    model = engine_model(folder, name, dtype)
+    if schedule == "whole":
+        steps, where = traces.whole(seqs)
+        max_tokens = 256
+    elif schedule == "tail":
+        steps, where = traces.tail_decoded(seqs)
+        max_tokens = 256
+    elif schedule == "portions":
+        steps, where = traces.portions(seqs, seed=3)
+        max_tokens = 256
+    else:
+        steps, where, peak = traces.mixed(seqs, seed=5)
+        max_tokens = peak  # so few pages that finished requests' pages are handed out again
+    replay(model, steps, where, ref, dtype, max_tokens, page)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_graph_and_eager_decode_agree(tiny_folders, name):
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, torch.bfloat16)
+    model = engine_model(folder, name, torch.bfloat16)
+    steps, where = traces.tail_decoded(seqs)
+    a = replay(model, steps, where, ref, torch.bfloat16, 256, page, graphs=True)
+    assert a.runner._graphs, "decode steps did not replay a graph"
+    replay(model, steps, where, ref, torch.bfloat16, 256, page, graphs=False)
+
+
+def test_trace_run_program(tiny_folders, tmp_path):
+    """bin/trace_run as a user calls it: JSON lines in, <step>.f32 out, 'done <step>' after every step."""
+    name = "B"
+    folder = tiny_folders[name]
+    seqs = sequences(name)
+    steps, where, peak = traces.mixed(seqs, seed=11)
+    for dtype_name, dtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        ref = plain_logits(folder, name, dtype)
+        out_dir = tmp_path / dtype_name
+        proc = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype_name,
+                               "--out", str(out_dir), "--max-tokens", str(peak)],
+                              input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        vocab = TINY[name]["cfg"]["vocab_size"]
+        for step, w in zip(steps, where):
+            path = out_dir / f"{step['step']}.f32"
+            if not w:
+                assert not path.exists()
+                continue
+            got = torch.from_file(str(path), size=len(w) * vocab, dtype=torch.float32).view(len(w), vocab)
+            check(got, torch.stack([ref[rid][p] for rid, p in w]), dtype, f"trace_run step {step['step']}")
