@@ -199,7 +199,7 @@ class ModelRunner:
 
     def _ensure_pad(self) -> None:
         if not self._pad_ready:
-            self.manager.admit(PAD_REQUEST)
+            self.admit(PAD_REQUEST)  # through admit(): the slot's mirrored block table starts empty
             self.manager.reserve(PAD_REQUEST, 1)
             self._mirror(self.manager.get(PAD_REQUEST))
             self._pad_ready = True

@@ -113,7 +113,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, token_req: torch.T
     _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
     if token_req.numel() != n or block_table.dim() != 2:
         raise KernelRefused("rope_kv_write: token_req is per token, block_table is [requests, pages]")
-    if inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2:
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2):
         raise KernelRefused("rope_kv_write: inv_freq must hold rotary_dim/2 float32 values")
     page = k_cache.shape[1]
     if (k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
