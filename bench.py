@@ -1,0 +1,173 @@
+"""Decode and prefill throughput of the Llama-3.1-8B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  ``value`` is decoded tokens per second at batch 8 through the whole engine (scheduler,
+step function, captured graphs, sampling): every request is prefilled with 2,048 random token ids, then W untimed
+and K timed decode steps run (K = 2,048 takes the context from 2,048 to 4,096).  ``points`` holds the same at
+batch 1 and 64 over a shorter window of steps centred on context 3,072, the mean of 2,048..4,096.  ``prefill`` is
+one step of 2,048 prompt tokens of one request; ``roofline`` is the bytes a decode step must read (every weight
+once, the cache of the live requests) over its time, against 8 TB/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_GBPS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+SHAPE_8B = dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+                num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=131072,
+                rope_scaling=dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192),
+                tie_word_embeddings=False)
+
+
+def weight_bytes(c, esize: int) -> int:
+    """Bytes of every weight a decode step reads once: the layers, the last norm and the head (an embedding row per
+    token is negligible and left out)."""
+    per_layer = ((c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * c.hidden_size
+                 + c.hidden_size * c.num_attention_heads * c.head_dim + 3 * c.intermediate_size * c.hidden_size + 2 * c.hidden_size)
+    return (c.num_hidden_layers * per_layer + c.hidden_size + c.vocab_size * c.hidden_size) * esize
+
+
+def kv_bytes_per_token(c, esize: int) -> int:
+    return c.num_hidden_layers * 2 * c.num_key_value_heads * c.head_dim * esize
+
+
+def prefill_flops(c, n: int, rows_with_logits: int) -> float:
+    per_layer = ((c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * c.hidden_size
+                 + c.hidden_size * c.num_attention_heads * c.head_dim + 3 * c.intermediate_size * c.hidden_size)
+    linear = 2.0 * n * c.num_hidden_layers * per_layer + 2.0 * rows_with_logits * c.vocab_size * c.hidden_size
+    attention = c.num_hidden_layers * 4.0 * c.num_attention_heads * c.head_dim * (n * (n + 1) / 2)
+    return linear + attention
+
+
+def decode_run(model, cfg, batch: int, prompt_len: int, first_ctx: int, steps: int, warmup: int, block_size: int, seed: int):
+    """-> (seconds for ``steps`` decode steps, context at the first and after the last timed step)."""
+    import torch
+
+    from nanospec_amd import Engine, EngineConfig, SamplingParams
+
+    total = first_ctx + warmup + steps + 1
+    blocks = batch * -(-(total + 1) // block_size) + 2
+    eng = Engine(model, EngineConfig(num_blocks=blocks, block_size=block_size, max_admit=batch, max_running=batch,
+                                     max_step_tokens=2048, prefill_chunk=2048, max_seq_len=total + block_size))
+    g = torch.Generator().manual_seed(seed)
+    # a prompt of ``first_ctx`` tokens puts the first decode step at that context
+    prompts = torch.randint(0, cfg.vocab_size, (batch, first_ctx), generator=g).tolist()
+    reqs = [eng.add(p, SamplingParams(max_tokens=warmup + steps + 1)) for p in prompts]
+    while any(r.computed < first_ctx for r in reqs):
+        eng.step()  # prefill in portions of at most 2,048 tokens
+    for _ in range(warmup):
+        eng.step()
+    eng.runner.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.step()
+    eng.runner.synchronize()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(len(r.out_tokens) == 1 + warmup + steps for r in reqs), "a decode step did not produce one token per request"
+    assert eng.runner.last_used_graph, "decode steps did not replay a captured graph"
+    ctx0 = first_ctx + 1 + warmup
+    del eng
+    torch.cuda.empty_cache()
+    return dt, ctx0, ctx0 + steps
+
+
+def prefill_run(model, cfg, n_tokens: int, block_size: int, reps: int = 3):
+    import torch
+
+    from nanospec_amd.engine.replay import Replayer
+
+    rep = Replayer(model, n_tokens + 64, page_size=block_size, use_graphs=False)
+    toks = torch.randint(0, cfg.vocab_size, (n_tokens,), generator=torch.Generator().manual_seed(7)).tolist()
+    best = None
+    for i in range(reps + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        rep.step([{"id": f"p{i}", "tokens": toks, "want": [n_tokens - 1]}], [f"p{i}"])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i and (best is None or dt < best):
+            best = dt  # the first pass warms the library's kernel selection
+    del rep
+    torch.cuda.empty_cache()
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2048)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU; this engine has no multi-GPU path (--gpus must be 1)")
+        return 2
+
+    import torch
+
+    from nanospec_amd import LlamaConfig
+    from nanospec_amd.loader import random_model
+
+    shape = dict(SHAPE_8B)
+    full_layers = shape["num_hidden_layers"]
+    if a.layers:
+        shape["num_hidden_layers"] = a.layers
+    cfg = LlamaConfig.from_hf(dict(model_type="llama", **{k: v for k, v in shape.items() if k != "rope_scaling"},
+                                   rope_scaling=dict(rope_type="llama3", **shape["rope_scaling"])))
+    dtype = torch.bfloat16 if a.dtype == "bf16" else torch.float32
+    esize = 2 if a.dtype == "bf16" else 4
+    model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
+    block, prompt, ctx_end = 16, 2048, 4096
+
+    steps = a.steps
+    dt, ctx0, ctx1 = decode_run(model, cfg, a.batch, prompt, prompt, steps, a.warmup, block, seed=1)
+    ms = 1000 * dt / steps
+    value = a.batch * steps / dt
+    mean_ctx = (ctx0 + ctx1 - 1) / 2
+    step_bytes = weight_bytes(cfg, esize) + a.batch * mean_ctx * kv_bytes_per_token(cfg, esize)
+    achieved = step_bytes / (dt / steps) / 1e9
+
+    p_tokens = 2048
+    p_dt = prefill_run(model, cfg, p_tokens, block)
+    p_frac = prefill_flops(cfg, p_tokens, 1) / p_dt / PEAK_FLOPS[a.dtype]
+
+    points = {}
+    if not a.no_points:
+        k = min(steps, 256)
+        for b in (1, 64):
+            d, _, _ = decode_run(model, cfg, b, prompt, 3072 - k // 2 - a.warmup - 1, k, a.warmup, block, seed=2 + b)
+            points[f"decode_b{b}"] = round(b * k / d, 1)
+
+    line = {
+        "metric": "decode tok/s at bs 8, ctx 2048->4096 (Llama-3.1-8B shape, bf16); prefill tok/s @2048 tok",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": a.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
+        "config": {"model": "Llama-3.1-8B shape", "layers": shape["num_hidden_layers"], "layers_of_shape": full_layers,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": prompt, "ctx_first_step": ctx0,
+                   "ctx_last_step": ctx1 - 1, "page_size": block, "parallelism": "single GPU", "graphs": True},
+        "prefill": {"value": round(p_tokens / p_dt, 1), "tokens": p_tokens, "ms": round(1000 * p_dt, 3), "frac": round(p_frac, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

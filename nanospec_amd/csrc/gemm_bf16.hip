@@ -43,6 +43,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(OutT* __restric
   const int per = (steps + WAVES - 1) / WAVES;
   const int ks0 = wave * per * 128;
   const int ks1 = min(K, ks0 + per * 128);
+  const int n_full = ks1 > ks0 ? (ks1 - ks0) / 128 : 0;  // super-steps with all 128 k inside K
 
   f32x4 acc[NACC][MT];
 #pragma unroll
@@ -51,24 +52,59 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(OutT* __restric
     for (int mt = 0; mt < MT; ++mt) acc[a][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  for (int ks = ks0; ks < ks1; ks += 128) {
+  // One super-step of operands: 4 fragments of w (and w2) and 4 per token tile of x.
+  struct Stage {
     bf16x8 wf[NACC][4], xf[MT][4];
+  };
+  auto load = [&](Stage& st, int ks) {
+    const int kk = ks + g * 32;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int kk = ks + g * 32 + i * 8;
-      const bool ok = kk < K;
-      wf[0][i] = ok ? load8(wrow + kk) : zero;
-      if (EPI == EPI_SILU_MUL) wf[NACC - 1][i] = ok ? load8(w2row + kk) : zero;
+      st.wf[0][i] = load8(wrow + kk + i * 8);
+      if (EPI == EPI_SILU_MUL) st.wf[NACC - 1][i] = load8(w2row + kk + i * 8);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xf[mt][i] = ok ? load8(xrow[mt] + kk) : zero;
+      for (int mt = 0; mt < MT; ++mt) st.xf[mt][i] = load8(xrow[mt] + kk + i * 8);
     }
+  };
+  auto mma = [&](const Stage& st) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int a = 0; a < NACC; ++a)
-          acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][i], xf[mt][i], acc[a][mt], 0, 0, 0);
+          acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.wf[a][i], st.xf[mt][i], acc[a][mt], 0, 0, 0);
+  };
+
+  // Full super-steps, two in flight: the loads of the next one are issued before the products of this one.
+  Stage s0, s1;
+  int ks = ks0;
+  if (n_full > 0) load(s0, ks);
+  int left = n_full;
+  while (left >= 2) {
+    load(s1, ks + 128);
+    mma(s0);
+    if (left > 2) load(s0, ks + 256);
+    mma(s1);
+    ks += 256;
+    left -= 2;
+  }
+  if (left == 1) {
+    mma(s0);
+    ks += 128;
+  }
+  // The ragged end of K: 8-element pieces beyond K are zero.
+  if (ks < ks1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kk = ks + g * 32 + i * 8;
+      const bool ok = kk < K;
+      s0.wf[0][i] = ok ? load8(wrow + kk) : zero;
+      if (EPI == EPI_SILU_MUL) s0.wf[NACC - 1][i] = ok ? load8(w2row + kk) : zero;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) s0.xf[mt][i] = ok ? load8(xrow[mt] + kk) : zero;
+    }
+    mma(s0);
   }
 
   // acc[a][mt][j] is the sum for w row n0 + 4 g + j and token 16 mt + r.
@@ -95,6 +131,152 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(OutT* __restric
     }
     out[(size_t)m * out_stride + n] = (OutT)s;
   }
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// The same product from weights that were re-laid at load time into the order in which the matrix
+// instruction wants them ("tiled" layout), so that every load of a wave is one contiguous kilobyte:
+//   wt[row tile rt][k tile kt][i = 0..3][lane = 16 g + r][e = 0..7] = w[16 rt + r][128 kt + 32 g + 8 i + e]
+// rows padded to a multiple of 16 and k to a multiple of 128 with zeros.  A workgroup owns one row tile;
+// its waves take the k tiles in turn (wave v takes kt = v, v + WAVES, ...), so the workgroup as a whole
+// walks through contiguous memory.  x is read as before; pieces of x beyond K are zero.
+// ------------------------------------------------------------------------------------------------
+template <int MT, int WAVES, int EPI, typename OutT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict__ out, const bf16_t* __restrict__ x,
+                                                                 const bf16_t* __restrict__ wt,
+                                                                 const bf16_t* __restrict__ wt2, int M, int N, int K,
+                                                                 int x_stride, int out_stride) {
+  constexpr int NACC = EPI == EPI_SILU_MUL ? 2 : 1;
+  __shared__ float red[WAVES][NACC * MT][256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int KT = (K + 127) / 128;
+  const bf16_t* wbase = wt + (size_t)blockIdx.x * KT * 2048 + lane * 8;
+  const bf16_t* w2base = EPI == EPI_SILU_MUL ? wt2 + (size_t)blockIdx.x * KT * 2048 + lane * 8 : nullptr;
+  const bf16_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + (size_t)min(mt * 16 + r, M - 1) * x_stride + g * 32;
+
+  f32x4 acc[NACC][MT];
+#pragma unroll
+  for (int a = 0; a < NACC; ++a)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[a][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  struct Stage {
+    bf16x8 wf[NACC][4], xf[MT][4];
+  };
+  auto load = [&](Stage& st, int kt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      st.wf[0][i] = load8(wbase + (size_t)kt * 2048 + i * 512);
+      if (EPI == EPI_SILU_MUL) st.wf[NACC - 1][i] = load8(w2base + (size_t)kt * 2048 + i * 512);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) st.xf[mt][i] = load8(xrow[mt] + kt * 128 + i * 8);
+    }
+  };
+  auto mma = [&](const Stage& st) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+          acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.wf[a][i], st.xf[mt][i], acc[a][mt], 0, 0, 0);
+  };
+
+  const int kt_full = K / 128;  // k tiles that x covers wholly
+  Stage s0, s1;
+  int kt = wave;
+  if (kt < kt_full) load(s0, kt);
+  while (kt + WAVES < kt_full) {
+    load(s1, kt + WAVES);
+    mma(s0);
+    if (kt + 2 * WAVES < kt_full) load(s0, kt + 2 * WAVES);
+    mma(s1);
+    kt += 2 * WAVES;
+  }
+  if (kt < kt_full) {
+    mma(s0);
+    kt += WAVES;
+  }
+  if (kt == kt_full && kt_full < KT) {  // the ragged end of K belongs to exactly one wave
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = kt * 128 + g * 32 + i * 8 < K;
+      s0.wf[0][i] = load8(wbase + (size_t)kt * 2048 + i * 512);
+      if (EPI == EPI_SILU_MUL) s0.wf[NACC - 1][i] = load8(w2base + (size_t)kt * 2048 + i * 512);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) s0.xf[mt][i] = ok ? load8(xrow[mt] + kt * 128 + i * 8) : zero;
+    }
+    mma(s0);
+  }
+
+#pragma unroll
+  for (int a = 0; a < NACC; ++a)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) red[wave][a * MT + mt][lane * 4 + j] = acc[a][mt][j];
+  __syncthreads();
+  for (int e = threadIdx.x; e < MT * 256; e += WAVES * 64) {
+    const int mt = e >> 8, le = e & 255;
+    const int l = le >> 2, j = le & 3;
+    const int n = n0 + (l >> 4) * 4 + j, m = mt * 16 + (l & 15);
+    if (n >= N || m >= M) continue;
+    float s = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) s += red[wv][mt][le];
+    if (EPI == EPI_SILU_MUL) {
+      float u = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) u += red[wv][MT + mt][le];
+      s = s / (1.f + expf(-s)) * u;
+    }
+    out[(size_t)m * out_stride + n] = (OutT)s;
+  }
+}
+
+template <int MT, int WAVES>
+static int launch_tiled(void* out, const void* x, const void* w, const void* w2, int M, int N, int K, int x_stride,
+                        int out_stride, int epi, int out_f32, hipStream_t stream) {
+  const int grid = (N + 15) / 16;
+  const bf16_t* xb = (const bf16_t*)x;
+  const bf16_t* wb = (const bf16_t*)w;
+  const bf16_t* w2b = (const bf16_t*)w2;
+  if (epi == EPI_SILU_MUL) {
+    if (out_f32) return NS_ERR_UNSUPPORTED;
+    gemm_tiled_kernel<MT, WAVES, EPI_SILU_MUL, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, w2b, M, N, K, x_stride, out_stride);
+  } else if (out_f32) {
+    gemm_tiled_kernel<MT, WAVES, EPI_STORE, float><<<grid, WAVES * 64, 0, stream>>>((float*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride);
+  } else {
+    gemm_tiled_kernel<MT, WAVES, EPI_STORE, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride);
+  }
+  return ns_launch_status();
+}
+
+// wt (and wt2) in the tiled layout described above; N and K are the sizes of the plain matrix.
+extern "C" int ns_gemm_tiled_bf16(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
+                                  int x_stride, int out_stride, int epi, int out_f32, int waves, hipStream_t stream) {
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
+  if (epi == EPI_SILU_MUL && !wt2) return NS_ERR_BAD_ARG;
+  const int mt = (M + 15) / 16;
+#define NS_TILED(MTV)                                                                                               \
+  case MTV:                                                                                                         \
+    return waves == 8 ? launch_tiled<MTV, 8>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, stream)  \
+         : waves == 2 ? launch_tiled<MTV, 2>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, stream)  \
+                      : launch_tiled<MTV, 4>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, stream);
+  switch (mt) {
+    NS_TILED(1)
+    NS_TILED(2)
+    NS_TILED(3)
+    NS_TILED(4)
+  }
+#undef NS_TILED
+  return NS_ERR_BAD_ARG;
 }
 
 template <int MT, int WAVES>

@@ -199,6 +199,63 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, w2: torch.Tensor | None = No
     return out
 
 
+class TiledWeight:
+    """A bfloat16 weight matrix [N, K] re-laid for the streaming matrix-core kernel:
+    wt[rt][kt][i][lane = 16 g + r][e] = w[16 rt + r][128 kt + 32 g + 8 i + e], rows padded to a multiple of 16 and
+    k to a multiple of 128 with zeros, so that every load of a wave is one contiguous kilobyte."""
+
+    def __init__(self, w: torch.Tensor) -> None:
+        if w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_cuda:
+            raise KernelRefused("TiledWeight takes a bfloat16 matrix on the GPU")
+        self.n, self.k = w.shape
+        n_pad, k_pad = -(-self.n // 16) * 16, -(-self.k // 128) * 128
+        if (n_pad, k_pad) != (self.n, self.k):
+            wp = torch.zeros((n_pad, k_pad), dtype=w.dtype, device=w.device)
+            wp[: self.n, : self.k] = w
+        else:
+            wp = w
+        # (rt, r, kt, g, i, e) -> (rt, kt, i, g, r, e)
+        self.data = wp.view(n_pad // 16, 16, k_pad // 128, 4, 4, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+
+    def rows(self, start: int, stop: int) -> "TiledWeight":
+        """The sub-matrix of rows [start, stop); both must be multiples of 16 (or stop the last row)."""
+        if start % 16 or (stop % 16 and stop != self.n):
+            raise KernelRefused("row slices of a tiled weight start and end at multiples of 16")
+        out = object.__new__(TiledWeight)
+        out.n, out.k = stop - start, self.k
+        out.data = self.data[start // 16 : -(-stop // 16)]
+        return out
+
+
+def tiled_takes(x: torch.Tensor, k: int) -> bool:
+    return (x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and k % 8 == 0 and x.stride(0) % 8 == 0
+            and x.stride(1) == 1 and x.data_ptr() % 16 == 0)
+
+
+def linear_tiled(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
+                 out_f32: bool = False, waves: int = 0) -> torch.Tensor:
+    """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T)."""
+    _gpu(x, out)
+    if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k):
+        raise KernelRefused(f"linear_tiled takes bfloat16 x [rows <= {SKINNY_MAX_ROWS}, {w.k}] with an inner size that is a "
+                            f"multiple of 8; got {tuple(x.shape)} {x.dtype}")
+    m = x.shape[0]
+    want = torch.float32 if out_f32 else x.dtype
+    if out is None:
+        out = torch.empty((m, w.n), dtype=want, device=x.device)
+    if out.shape != (m, w.n) or out.dtype != want or out.stride(1) != 1:
+        raise KernelRefused("linear_tiled: out has the wrong shape or dtype")
+    if w2 is not None and (w2.n != w.n or w2.k != w.k):
+        raise KernelRefused("linear_tiled: w2 must match w")
+    if waves == 0:
+        waves = 8 if w.k >= 8192 or (w.n // 16 < 512 and w.k >= 2048) else 4
+    _check(build.core().ns_gemm_tiled_bf16(_ptr(out), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None), c_int(m),
+                                           c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
+                                           c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(waves), _stream()),
+           "linear_tiled")
+    return out
+
+
 # ------------------------------------------------------------------------------------------------ attention
 
 

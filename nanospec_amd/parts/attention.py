@@ -14,7 +14,7 @@ import torch
 
 from ..kernels import ops
 from . import registry
-from .linear import linear
+from .linear import LinearWeight
 from .needs import PagedNeed
 
 
@@ -28,8 +28,8 @@ class Attention:
         self.position = registry.build("position", spec.position, prefix)
         if self.position.rotary_dim > spec.head_dim:
             raise ValueError("the rotary part of a head cannot be wider than the head")
-        self.wqkv: torch.Tensor | None = None
-        self.wo: torch.Tensor | None = None
+        self.wqkv: LinearWeight | None = None
+        self.wo: LinearWeight | None = None
 
     @property
     def _names(self):
@@ -51,13 +51,14 @@ class Attention:
         s = self.spec
         q, k, v, o = self._names
         rows = (s.heads + 2 * s.kv_heads) * s.head_dim
-        self.wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
+        wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
         at = 0
         for name in (q, k, v):
             t = get(name)
-            self.wqkv[at : at + t.shape[0]].copy_(t)
+            wqkv[at : at + t.shape[0]].copy_(t)
             at += t.shape[0]
-        self.wo = get(o).to(device=device, dtype=dtype).contiguous()
+        self.wqkv = LinearWeight(wqkv)
+        self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous())
         self.position.load(get, dtype, device)
 
     def cache_need(self):
@@ -69,7 +70,7 @@ class Attention:
         pos = self.position
         if pos.max_positions is not None and ctx.max_position >= pos.max_positions:
             raise ValueError(f"position {ctx.max_position} is beyond the model's {pos.max_positions} positions")
-        qkv = linear(x, self.wqkv, out=ctx.arena.take(((n, self.wqkv.shape[0])), x.dtype))
+        qkv = self.wqkv(x, out=ctx.arena.take((n, self.wqkv.n), x.dtype))
         table = ctx.block_tables[cache.group]
         ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
                           s.head_dim, pos.rotary_dim, write_kv=owns_cache)
@@ -84,7 +85,7 @@ class Attention:
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)
-        return linear(att, self.wo, out=out)
+        return self.wo(att, out=out)
 
 
 registry.register("mixer", "attention", Attention)

@@ -1,10 +1,14 @@
-"""x @ W^T for the parts, choosing the kernel by precision and row count.
+"""x @ W^T for the parts: ``LinearWeight`` holds a weight matrix and chooses the kernel by precision and row count.
 
-float32: always the plain tiled kernel with 32-bit fused multiply-adds in a fixed order (the true
-32-bit path; no matrix-core mode of reduced precision is ever used).
-bfloat16: up to 64 rows the hand-written matrix-core kernel that streams W once; beyond that the
-platform's GEMM library, as the reference's nn.Linear does (model/llama.py:168-171), except for
-32-bit results (logits), which run through the streaming kernel in slices of 64 rows.
+float32: always the plain tiled kernel with 32-bit fused multiply-adds in a fixed order (the true 32-bit path; no
+matrix-core mode of reduced precision is ever used).
+
+bfloat16: decode and short portions (up to ``STREAM_ROWS`` rows) run the hand-written matrix-core kernel that streams
+the weights once; it reads them in a layout re-laid at load time (``kernels.ops.TiledWeight``) in which every load
+of a wave is one contiguous kilobyte.  More rows go to the platform's GEMM library on the plain layout, as the
+reference's nn.Linear does (model/llama.py:168-171).  32-bit results (logits) always come from the streaming kernel,
+in slices of 64 rows, so that no logit is rounded to bfloat16.  Both layouts are kept in memory unless
+``keep_plain=False``.
 """
 
 from __future__ import annotations
@@ -13,37 +17,57 @@ import torch
 
 from ..kernels import ops
 
-
-def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False) -> torch.Tensor:
-    if x.dtype == torch.float32:
-        return ops.linear_generic(x, w, out=out, out_f32=out_f32)
-    if not ops.skinny_takes(x[:1], w):
-        if x.shape[0] > ops.SKINNY_MAX_ROWS and not out_f32 and w.shape[1] % 8 == 0:
-            return _library(x, w, out)
-        return ops.linear_generic(x, w, out=out, out_f32=out_f32)
-    m = x.shape[0]
-    if m <= ops.SKINNY_MAX_ROWS:
-        return ops.linear_skinny(x, w, out=out, out_f32=out_f32)
-    if not out_f32:
-        return _library(x, w, out)
-    if out is None:
-        out = torch.empty((m, w.shape[0]), dtype=torch.float32, device=x.device)
-    for s in range(0, m, ops.SKINNY_MAX_ROWS):
-        e = min(m, s + ops.SKINNY_MAX_ROWS)
-        ops.linear_skinny(x[s:e], w, out=out[s:e], out_f32=True)
-    return out
+STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured (see profiles/)
 
 
-def _library(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
-    if out is None:
-        return torch.matmul(x, w.t())
-    return torch.matmul(x, w.t(), out=out)
+class LinearWeight:
+    def __init__(self, w: torch.Tensor, keep_plain: bool = True) -> None:
+        """``w``: [out, in] on the GPU in the compute dtype."""
+        self.n, self.k = w.shape
+        self.dtype = w.dtype
+        self.plain = w if (keep_plain or w.dtype != torch.bfloat16 or self.k % 8) else None
+        self.tiled = ops.TiledWeight(w) if (w.dtype == torch.bfloat16 and self.k % 8 == 0) else None
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False) -> torch.Tensor:
+        if x.dtype != self.dtype:
+            raise ops.KernelRefused(f"linear: input is {x.dtype}, the weight {self.dtype}")
+        if self.dtype == torch.float32 or self.tiled is None or not ops.tiled_takes(x[:1], self.k):
+            return ops.linear_generic(x, self.plain, out=out, out_f32=out_f32)
+        m = x.shape[0]
+        if m <= STREAM_ROWS or (m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None)):
+            return ops.linear_tiled(x, self.tiled, out=out, out_f32=out_f32)
+        if not out_f32 and self.plain is not None:
+            return torch.matmul(x, self.plain.t()) if out is None else torch.matmul(x, self.plain.t(), out=out)
+        if out is None:
+            out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
+        for s in range(0, m, ops.SKINNY_MAX_ROWS):
+            e = min(m, s + ops.SKINNY_MAX_ROWS)
+            ops.linear_tiled(x[s:e], self.tiled, out=out[s:e], out_f32=out_f32)
+        return out
 
 
-def swiglu_up(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor | None = None, scratch=None) -> torch.Tensor:
-    """silu(x @ Wg^T) * (x @ Wu^T) for gate_up = [Wg; Wu] of shape [2 I, H]."""
-    inter = gate_up.shape[0] // 2
-    if x.dtype == torch.bfloat16 and x.shape[0] <= ops.SKINNY_MAX_ROWS and ops.skinny_takes(x, gate_up):
-        return ops.linear_skinny(x, gate_up[:inter], w2=gate_up[inter:], out=out)
-    gu = linear(x, gate_up, out=scratch)
-    return ops.silu_mul(gu, out=out)
+class GatedWeights:
+    """Gate and up matrices of a gated feed-forward: silu(x @ Wg^T) * (x @ Wu^T) in one pass over x."""
+
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_plain: bool = True) -> None:
+        self.inter, self.k = gate.shape
+        self.dtype = gate.dtype
+        fast = gate.dtype == torch.bfloat16 and self.k % 8 == 0
+        self.tiled = (ops.TiledWeight(gate), ops.TiledWeight(up)) if fast else None
+        self.stacked = torch.cat([gate, up]) if (keep_plain or not fast) else None  # [2 I, K] for the two-kernel path
+
+    def __call__(self, ctx, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        m = x.shape[0]
+        if self.tiled is not None and ops.tiled_takes(x[:1], self.k) and (m <= STREAM_ROWS or (self.stacked is None and m <= ops.SKINNY_MAX_ROWS)):
+            return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
+        if self.stacked is None:
+            for s in range(0, m, ops.SKINNY_MAX_ROWS):
+                e = min(m, s + ops.SKINNY_MAX_ROWS)
+                ops.linear_tiled(x[s:e], self.tiled[0], w2=self.tiled[1], out=out[s:e])
+            return out
+        gu = ctx.arena.take((m, 2 * self.inter), x.dtype)
+        if self.dtype == torch.float32 or self.k % 8:
+            ops.linear_generic(x, self.stacked, out=gu)
+        else:
+            torch.matmul(x, self.stacked.t(), out=gu)
+        return ops.silu_mul(gu, out=out)

@@ -8,7 +8,7 @@ import torch
 from ..kernels import ops
 from ..weights import source as wsource
 from . import registry
-from .linear import linear
+from .linear import LinearWeight
 from .needs import PagedNeed, StateNeed
 
 
@@ -33,7 +33,7 @@ class DecoderModel:
         self.layers = _build_layers(spec)
         self.final_norm = registry.build("norm", spec.final_norm, spec.final_norm_name)
         self.embed: torch.Tensor | None = None
-        self.head: torch.Tensor | None = None
+        self.head: LinearWeight | None = None
         self.dtype = self.device = None
         # what every entry of the run order keeps in the cache
         self.cache_needs = [self.layers[c.layer].cache_need() if c.cache_from is None else None for c in spec.run_order]
@@ -56,9 +56,9 @@ class DecoderModel:
         get = source.get
         self.embed = get(spec.embed_name).to(device=device, dtype=dtype).contiguous()
         if spec.head_name in source.names():
-            self.head = get(spec.head_name).to(device=device, dtype=dtype).contiguous()
+            self.head = LinearWeight(get(spec.head_name).to(device=device, dtype=dtype).contiguous(), keep_plain=False)
         else:
-            self.head = self.embed  # one storage
+            self.head = LinearWeight(self.embed, keep_plain=False)  # the embedding table is the head
         for layer in self.layers:
             layer.load(get, dtype, device)
         self.final_norm.load(get, dtype, device)
@@ -85,4 +85,4 @@ class DecoderModel:
         (reference: model/llama.py:284-286, engine/engine.py:382)."""
         n = rows.numel()
         h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
-        return linear(h, self.head, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True)
+        return self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True)

@@ -95,6 +95,29 @@ def test_linear_skinny(m, n, k):
     assert ulps_of_row_max(act.cpu(), want).max() <= 1.0
 
 
+@pytest.mark.parametrize("m", [1, 7, 16, 33, 64])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064), (16, 8), (4096, 14336)])
+def test_linear_tiled(m, n, k):
+    """The streaming kernel on weights in the tiled layout: sizes that are no multiples of the tile, every wave count."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m, k, dtype=torch.bfloat16, device=DEV)
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    wt, wt2 = ops.TiledWeight(w), ops.TiledWeight(w2)
+    ref = x.cpu().float() @ w.cpu().float().T
+    for waves in (2, 4, 8):
+        out = ops.linear_tiled(x, wt, out_f32=True, waves=waves)
+        torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
+    assert ulps_of_row_max(ops.linear_tiled(x, wt).cpu(), ref).max() <= 1.0
+    u = x.cpu().float() @ w2.cpu().float().T
+    act = ops.linear_tiled(x, wt, w2=wt2)
+    assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0
+    if n >= 64:  # a slice of rows, as the stacked gate/up and q/k/v matrices are used
+        part = ops.linear_tiled(x, wt.rows(16, 48), out_f32=True)
+        torch.testing.assert_close(part.cpu(), ref[:, 16:48], rtol=1e-4, atol=1e-3 * math.sqrt(k))
+
+
 def test_linear_skinny_refuses():
     ops = _ops()
     from nanospec_amd.kernels import KernelRefused
