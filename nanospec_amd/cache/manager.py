@@ -41,6 +41,7 @@ class RequestCache:
     reserved: int = 0
     length: int = 0
     first_kept: list[int] = field(default_factory=list)  # per group: first table index not released
+    held: list[int] = field(default_factory=list)  # per group: pages held now
 
 
 class CacheManager:
@@ -102,7 +103,8 @@ class CacheManager:
     def admit(self, req_id) -> RequestCache:
         if req_id in self._live:
             raise ValueError(f"request {req_id!r} is already live")
-        rc = RequestCache(req_id, self.slots.take(), [[] for _ in self.groups], first_kept=[0] * len(self.groups))
+        rc = RequestCache(req_id, self.slots.take(), [[] for _ in self.groups], first_kept=[0] * len(self.groups),
+                          held=[0] * len(self.groups))
         self._live[req_id] = rc
         return rc
 
@@ -119,6 +121,7 @@ class CacheManager:
                 )
         for g, need in enumerate(missing):
             rc.tables[g].extend(self.pools[g].take(need))
+            rc.held[g] += need
         rc.reserved = max(rc.reserved, rc.length + n_tokens)
         return rc
 
@@ -134,6 +137,7 @@ class CacheManager:
             gone = [p for p in rc.tables[g][rc.first_kept[g]:keep_from] if p != RELEASED]
             if gone:
                 self.pools[g].give(gone)
+                rc.held[g] -= len(gone)
             for i in range(rc.first_kept[g], keep_from):
                 rc.tables[g][i] = RELEASED
             rc.first_kept[g] = max(rc.first_kept[g], keep_from)
@@ -144,6 +148,7 @@ class CacheManager:
         for g, table in enumerate(rc.tables):
             self.pools[g].give([p for p in table if p != RELEASED])
             table.clear()
+            rc.held[g] = 0
         self.slots.give(rc.slot)
         rc.reserved = rc.length = 0
 
@@ -159,6 +164,7 @@ class CacheManager:
                 assert len(rc.tables[g]) == self.pages_for(rc.reserved), (rc.req_id, g, rc.tables[g], rc.reserved)
                 assert all(p == RELEASED for p in rc.tables[g][: rc.first_kept[g]])
                 assert all(p != RELEASED for p in rc.tables[g][rc.first_kept[g]:])
+                assert rc.held[g] == sum(1 for p in rc.tables[g] if p != RELEASED)
             assert sorted(seen) == list(range(pool.num_pages)), f"group {g}: a page is lost or held twice"
         held = self.slots.free_slots() + [rc.slot for rc in self._live.values()]
         assert sorted(held) == list(range(self.slots.num_slots)), "a state slot is lost or held twice"

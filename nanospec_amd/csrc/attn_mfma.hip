@@ -20,7 +20,7 @@
 //
 // Query at position p sees keys max(0, p - window + 1) .. p.  Scores, soft-max and sums are 32-bit.
 // With splits > 1 the keys of a tile are cut into `splits` contiguous ranges of whole 32-key blocks;
-// each range writes its un-normalised output, maximum and sum, and ns_attn_mfma_reduce joins them.
+// each range writes its un-normalised output, maximum and sum, and a second small kernel joins them.
 #include "common.h"
 
 #ifndef NS_HEAD_DIM
@@ -89,9 +89,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const int lo = (col_ok && a.window > 0) ? max(0, pos - a.window + 1) : 0;
   const int whi = wave_max_i(pos) + 1;                    // keys [wlo, whi) are seen by some column
   const int wlo = wave_min_i(col_ok ? lo : 0x7fffffff);
-  if (whi <= 0) return;
-
-  int kb0 = wlo / 32, kb1 = (whi + 31) / 32;
+  // (a tile always holds a column; if it did not, the wave would still have to reach the counter below)
+  int kb0 = whi > 0 ? wlo / 32 : 0, kb1 = whi > 0 ? (whi + 31) / 32 : 0;
   if (a.splits > 1) {
     const int per = (kb1 - kb0 + a.splits - 1) / a.splits;
     kb0 = kb0 + split * per;
@@ -191,17 +190,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 
   lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
-  if (!col_ok) return;
   // o[dt][j] is channel 16 dt + 4 g + j of column c
-  const size_t col = (size_t)(q0 + ti) * a.heads + head;
+  const size_t col = (size_t)(q0 + (col_ok ? ti : 0)) * a.heads + head;
   if (a.splits == 1) {
+    if (!col_ok) return;
     const float inv = 1.f / lsum;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       bf16x4 r = {(bf16_t)(o[dt][0] * inv), (bf16_t)(o[dt][1] * inv), (bf16_t)(o[dt][2] * inv), (bf16_t)(o[dt][3] * inv)};
       *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
     }
-  } else {
+  } else if (col_ok) {
     float* po = a.part_o + (col * a.splits + split) * HD;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
@@ -212,8 +211,9 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   }
 }
 
-// out[col] = sum_s o_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*), m* = max_s m_s; splits are joined in order.
-// One workgroup per (tile, head): it joins the columns of that head for the tile's tokens.
+// Joining the key ranges: out[col] = sum_s o_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*), m* = max_s m_s.
+// One wave per (tile, head) and token of the tile; lane s first holds range s (at most 64 ranges), so the maxima
+// and weights are formed by wave reductions, then the lanes split the channels and add the ranges in order.
 __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                                          const float* __restrict__ part_ml,
                                                          const int* __restrict__ tile_req, const int* __restrict__ tile_t0,
@@ -221,23 +221,28 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ ou
   const int b = tile_req[blockIdx.x], t0 = tile_t0[blockIdx.x], head = blockIdx.y;
   const int q0 = qo_indptr[b], n = qo_indptr[b + 1] - q0;
   const int t1 = min(n, t0 + 16 / hp);
+  const int lane = threadIdx.x;
   for (int ti = t0; ti < t1; ++ti) {
     const size_t col = (size_t)(q0 + ti) * heads + head;
     const float* ml = part_ml + col * splits * 2;
-    float mstar = -INFINITY;
-    for (int s = 0; s < splits; ++s) mstar = fmaxf(mstar, ml[s * 2]);
-    float l = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = ml[s * 2];
-      if (ms != -INFINITY) l += ml[s * 2 + 1] * exp2f(ms - mstar);
+    float ms = -INFINITY, ls = 0.f;
+    if (lane < splits) {
+      ms = ml[lane * 2];
+      ls = ml[lane * 2 + 1];
     }
-    for (int d = threadIdx.x; d < HD; d += 64) {
+    float mstar = ms;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, o, 64));
+    const float wgt = ms == -INFINITY ? 0.f : exp2f(ms - mstar);
+    float l = ls * wgt;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+    const float inv = 1.f / l;
+    for (int d = lane; d < HD; d += 64) {
       float acc = 0.f;
-      for (int s = 0; s < splits; ++s) {
-        const float ms = ml[s * 2];
-        if (ms != -INFINITY) acc += part_o[(col * splits + s) * HD + d] * exp2f(ms - mstar);
-      }
-      out[col * HD + d] = (bf16_t)(acc / l);
+      const float* po = part_o + col * splits * HD + d;
+      for (int s = 0; s < splits; ++s) acc += po[(size_t)s * HD] * __shfl(wgt, s, 64);
+      out[col * HD + d] = (bf16_t)(acc * inv);
     }
   }
 }
@@ -254,6 +259,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
       window < 0 || splits < 1 || (q_stride & 7))
     return NS_ERR_BAD_ARG;
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
+  if (splits > 64) return NS_ERR_BAD_ARG;
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
   AttnParams a;
   a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
@@ -267,7 +273,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const long blocks = (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
   attn_mfma_kernel<<<(unsigned)blocks, 256, 0, stream>>>(a);
-  int st = ns_launch_status();
+  const int st = ns_launch_status();
   if (st != NS_OK || splits == 1) return st;
   if (heads > 65535) return NS_ERR_BAD_ARG;
   attn_reduce_kernel<<<dim3(n_tiles, heads), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml, tile_req,

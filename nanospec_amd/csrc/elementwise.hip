@@ -60,11 +60,85 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, T* resid, const T* __restric
   }
 }
 
+// The same with 16-byte accesses and the row kept in registers between the two passes; for rows of a multiple
+// of 16 bytes and at most 4 pieces per thread.
+template <typename T, int MAXC>
+__global__ void rmsnorm_vec_kernel(T* __restrict__ out, T* resid, const T* __restrict__ x, const T* __restrict__ w,
+                                   const int* __restrict__ rows, int dim, float eps, int write_resid) {
+  constexpr int V = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const size_t r = rows ? (size_t)rows[i] : (size_t)i;
+  const vec_t* xr = x ? reinterpret_cast<const vec_t*>(x + r * dim) : nullptr;
+  vec_t* rr = resid ? reinterpret_cast<vec_t*>(resid + r * dim) : nullptr;
+  const int nvec = dim / V;
+  vec_t val[MAXC];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int idx = threadIdx.x + c * blockDim.x;
+    if (idx < nvec) {
+      vec_t a = rr ? rr[idx] : vec_t{};
+      if (xr) {
+        const vec_t b = xr[idx];
+        if (rr) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) a[e] = from_f<T>(to_f(a[e]) + to_f(b[e]));
+        } else {
+          a = b;
+        }
+      }
+      val[c] = a;
+#pragma unroll
+      for (int e = 0; e < V; ++e) ss += to_f(a[e]) * to_f(a[e]);
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rinv = rsqrtf(ss / (float)dim + eps);
+  vec_t* o = reinterpret_cast<vec_t*>(out + (size_t)i * dim);
+  const vec_t* wv = reinterpret_cast<const vec_t*>(w);
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int idx = threadIdx.x + c * blockDim.x;
+    if (idx < nvec) {
+      if (write_resid && rr && xr) rr[idx] = val[c];
+      const vec_t ww = wv[idx];
+      vec_t y;
+#pragma unroll
+      for (int e = 0; e < V; ++e) y[e] = from_f<T>(to_f(ww[e]) * round_to<T>(to_f(val[c][e]) * rinv));
+      o[idx] = y;
+    }
+  }
+}
+
+template <typename T>
+static bool launch_rmsnorm_vec(void* out, void* resid, const void* x, const void* w, const int* rows, int n_rows, int dim,
+                               float eps, int write_resid, hipStream_t stream) {
+  constexpr int V = 16 / sizeof(T);
+  if (dim % V) return false;
+  if (((uintptr_t)out | (uintptr_t)resid | (uintptr_t)x | (uintptr_t)w) & 15) return false;
+  const int nvec = dim / V;
+  int threads = ((nvec + 63) / 64) * 64;
+  if (threads > 1024) threads = 1024;
+  const int chunks = (nvec + threads - 1) / threads;
+  if (chunks > 4) return false;
+  if (chunks <= 1)
+    rmsnorm_vec_kernel<T, 1><<<n_rows, threads, 0, stream>>>((T*)out, (T*)resid, (const T*)x, (const T*)w, rows, dim, eps, write_resid);
+  else if (chunks == 2)
+    rmsnorm_vec_kernel<T, 2><<<n_rows, threads, 0, stream>>>((T*)out, (T*)resid, (const T*)x, (const T*)w, rows, dim, eps, write_resid);
+  else
+    rmsnorm_vec_kernel<T, 4><<<n_rows, threads, 0, stream>>>((T*)out, (T*)resid, (const T*)x, (const T*)w, rows, dim, eps, write_resid);
+  return true;
+}
+
 extern "C" int ns_rmsnorm(void* out, void* resid, const void* x, const void* w, const int* rows, int n_rows, int dim,
                           float eps, int write_resid, int dtype, hipStream_t stream) {
   if (n_rows <= 0 || dim <= 0 || (!resid && !x)) return NS_ERR_BAD_ARG;
   if (write_resid && rows) return NS_ERR_BAD_ARG;  // a gathered row may be named twice
   const int threads = dim >= 2048 ? 512 : 256;
+  if (dtype == NS_DTYPE_F32 && launch_rmsnorm_vec<float>(out, resid, x, w, rows, n_rows, dim, eps, write_resid, stream)) return ns_launch_status();
+  if (dtype == NS_DTYPE_BF16 && launch_rmsnorm_vec<bf16_t>(out, resid, x, w, rows, n_rows, dim, eps, write_resid, stream)) return ns_launch_status();
   if (dtype == NS_DTYPE_F32)
     rmsnorm_kernel<float><<<n_rows, threads, 0, stream>>>((float*)out, (float*)resid, (const float*)x, (const float*)w, rows, dim, eps, write_resid);
   else if (dtype == NS_DTYPE_BF16)
@@ -89,16 +163,22 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* _
                                const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
                                const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                int heads, int kv_heads, int hd, int rot, int page_size, int write_kv) {
+  extern __shared__ float cs[];  // cos[half] | sin[half] of this token's angles
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (size_t)t * row_stride;
   const int half = rot / 2;
   const float fpos = (float)pos;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const float ang = fpos * inv_freq[j];
+    cs[j] = cosf(ang);
+    cs[half + j] = sinf(ang);
+  }
+  __syncthreads();
   // q heads, in place
   for (int e = threadIdx.x; e < heads * half; e += blockDim.x) {
     const int h = e / half, j = e - h * half;
-    const float ang = fpos * inv_freq[j];
-    const float c = cosf(ang), s = sinf(ang);
+    const float c = cs[j], s = cs[half + j];
     T* p = row + h * hd;
     const float a = to_f(p[j]), b = to_f(p[j + half]);
     p[j] = from_f<T>(a * c - b * s);
@@ -116,8 +196,7 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* _
     float kv;
     if (d < rot) {
       const int j = d < half ? d : d - half;
-      const float ang = fpos * inv_freq[j];
-      const float c = cosf(ang), s = sinf(ang);
+      const float c = cs[j], s = cs[half + j];
       const float a = to_f(krow[h * hd + j]), b = to_f(krow[h * hd + j + half]);
       kv = d < half ? a * c - b * s : b * c + a * s;
     } else {
@@ -134,11 +213,13 @@ extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions,
                                 int write_kv, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || rot < 0 || rot > hd || (rot & 1) || page_size <= 0)
     return NS_ERR_BAD_ARG;
+  const int work = heads * (rot / 2) > kv_heads * hd ? heads * (rot / 2) : kv_heads * hd;
+  const int threads = work >= 1024 ? 1024 : work >= 512 ? 512 : 256;
   if (dtype == NS_DTYPE_F32)
-    rope_kv_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, row_stride, positions, token_req, block_table, table_stride,
+    rope_kv_kernel<float><<<n_tokens, threads, (size_t)(rot + 2) * sizeof(float), stream>>>((float*)qkv, row_stride, positions, token_req, block_table, table_stride,
                                                         inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
   else if (dtype == NS_DTYPE_BF16)
-    rope_kv_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, row_stride, positions, token_req, block_table, table_stride,
+    rope_kv_kernel<bf16_t><<<n_tokens, threads, (size_t)(rot + 2) * sizeof(float), stream>>>((bf16_t*)qkv, row_stride, positions, token_req, block_table, table_stride,
                                                          inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
   else
     return NS_ERR_UNSUPPORTED;
@@ -158,8 +239,34 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
   }
 }
 
+template <typename T>
+__global__ void silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, size_t total_vec) {
+  constexpr int V = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const int ivec = inter / V;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total_vec; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = e / ivec;
+    const int i = (int)(e - n * ivec);
+    const vec_t g = reinterpret_cast<const vec_t*>(gu + n * 2 * inter)[i];
+    const vec_t u = reinterpret_cast<const vec_t*>(gu + n * 2 * inter + inter)[i];
+    vec_t y;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const float gf = to_f(g[k]);
+      y[k] = from_f<T>(gf / (1.f + expf(-gf)) * to_f(u[k]));
+    }
+    reinterpret_cast<vec_t*>(out + n * inter)[i] = y;
+  }
+}
+
 extern "C" int ns_silu_mul(void* out, const void* gu, int n_rows, int inter, int dtype, hipStream_t stream) {
   if (n_rows <= 0 || inter <= 0) return NS_ERR_BAD_ARG;
+  if (dtype == NS_DTYPE_BF16 && inter % 8 == 0 && !(((uintptr_t)out | (uintptr_t)gu) & 15)) {
+    const size_t tv = (size_t)n_rows * (inter / 8);
+    const int nb = (int)((tv + 255) / 256 < 16384 ? (tv + 255) / 256 : 16384);
+    silu_mul_vec_kernel<bf16_t><<<nb, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, inter, tv);
+    return ns_launch_status();
+  }
   const size_t total = (size_t)n_rows * inter;
   const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
   if (dtype == NS_DTYPE_F32)

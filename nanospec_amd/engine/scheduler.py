@@ -114,16 +114,14 @@ class Scheduler:
         self.waiting.append(req)
 
     def _capacity(self, g: int) -> int:
-        held_by_others = 0
-        for rid in self.cache.live:
-            if not any(r.id == rid for r in self.running):
-                held_by_others += sum(1 for p in self.cache.get(rid).tables[g] if p >= 0)
+        ours = {r.id for r in self.running}
+        held_by_others = sum(self.cache.get(rid).held[g] for rid in self.cache.live if rid not in ours)
         return self.cache.pools[g].num_pages - held_by_others
 
     # ------------------------------------------------------------------ admission
 
     def _held(self, req: Request) -> list[int]:
-        return [sum(1 for p in t if p >= 0) for t in self.cache.get(req.id).tables]
+        return self.cache.get(req.id).held
 
     def _admit(self) -> list[Request]:
         groups = range(len(self.cache.groups))

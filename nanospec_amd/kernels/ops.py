@@ -298,7 +298,7 @@ def attention_mfma(q, out, k_cache, v_cache, tile_req, tile_t0, qo_indptr, kv_le
                    workspace: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
     """bfloat16 attention on the matrix cores for the tiles (request, first token) listed in ``tile_req`` /
     ``tile_t0``.  ``hp`` heads of a group times 16/hp tokens make a tile; ``splits`` > 1 cuts the keys of
-    every tile into that many ranges and needs ``workspace`` = (part_o, part_ml) float32 tensors."""
+    every tile into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
     if not mfma_attention_takes(q.dtype, head_dim, page):
         raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
@@ -309,8 +309,8 @@ def attention_mfma(q, out, k_cache, v_cache, tile_req, tile_t0, qo_indptr, kv_le
     n_tiles, n_tokens = tile_req.numel(), q.shape[0]
     po = pm = None
     if splits > 1:
-        if workspace is None:
-            raise KernelRefused("attention_mfma: splits > 1 needs a workspace")
+        if workspace is None or splits > 64:
+            raise KernelRefused("attention_mfma: 2 to 64 key ranges are taken, with a workspace")
         po, pm = workspace
         if po.dtype != torch.float32 or pm.dtype != torch.float32 or po.numel() < n_tokens * heads * splits * head_dim or pm.numel() < n_tokens * heads * splits * 2:
             raise KernelRefused("attention_mfma: workspace too small")
