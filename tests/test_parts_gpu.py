@@ -1,0 +1,264 @@
+"""Each kind of part alone against the plain function it implements, at sizes of its own; a model put together from
+parts in an unusual order (a layer run twice, an entry that reads another entry's cache); and a toy mixer with state of
+its own that is defined here, registered, built and stepped without touching the framework."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import ClassVar
+
+import pytest
+import torch
+
+import plain_llama as pl
+from tiny import ulps_of_row_max
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def make_ctx(lens, starts, tables, page, dtype, want=()):
+    """A StepContext for hand-made requests: tables[b] lists the pages of request b."""
+    import numpy as np
+
+    from nanospec_amd.engine.arena import Arena
+    from nanospec_amd.engine.context import BatchLayout, StepContext, count_tiles, fill_batch
+
+    tc, td = count_tiles(lens)
+    width = max(len(t) for t in tables)
+    layout = BatchLayout(sum(lens), len(lens), len(want), tc, td, 1, width)
+    host = np.zeros(layout.total, dtype=np.int32)
+    table = np.full((len(lens), width), -1, dtype=np.int32)
+    for b, t in enumerate(tables):
+        table[b, : len(t)] = t
+    fill_batch(host, layout, [0] * sum(lens), starts, lens, list(range(len(lens))), list(want), [table])
+    dev = torch.from_numpy(host).to(DEV)
+    max_kv = max(s + n for s, n in zip(starts, lens))
+    return StepContext(layout, dev, Arena(DEV), max_position=max_kv - 1, max_kv_len=max_kv)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_norm_part(dtype):
+    from nanospec_amd.config.spec import RMSNormSpec
+    from nanospec_amd.parts import build
+
+    torch.manual_seed(0)
+    part = build("norm", RMSNormSpec(dim=88, eps=2e-6), "x.norm.weight")
+    assert part.wanted() == {"x.norm.weight": ((88,), "norm")}
+    w = 1 + 0.1 * torch.randn(88)
+    part.load({"x.norm.weight": w}.__getitem__, dtype, DEV)
+    x = torch.randn(5, 88).to(dtype)
+    got = part.forward(None, resid=x.to(DEV))
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got.cpu().float(), pl.rms_norm(x, w.to(dtype), 2e-6).float(), **tol)
+
+
+def test_rope_part_frequencies():
+    from nanospec_amd.config.spec import RopeSpec
+    from nanospec_amd.parts import build
+
+    for scaling in (None, (8.0, 1.0, 4.0, 64), (32.0, 1.0, 4.0, 8192)):
+        part = build("position", RopeSpec(rotary_dim=48, theta=5e5, scaling=scaling, max_positions=512), "")
+        part.load(None, torch.float32, DEV)
+        s = None if scaling is None else dict(factor=scaling[0], low_freq_factor=scaling[1], high_freq_factor=scaling[2],
+                                              original_max_position_embeddings=scaling[3])
+        assert torch.equal(part.inv_freq.cpu(), pl.inverse_frequencies(48, 5e5, s))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_feed_forward_part(dtype):
+    from nanospec_amd.config.spec import SwiGLUSpec
+    from nanospec_amd.parts import build
+
+    torch.manual_seed(1)
+    part = build("ffn", SwiGLUSpec(hidden=72, intermediate=200), "l.mlp.")
+    ws = {"l.mlp.gate_proj.weight": torch.randn(200, 72) * 0.1, "l.mlp.up_proj.weight": torch.randn(200, 72) * 0.1,
+          "l.mlp.down_proj.weight": torch.randn(72, 200) * 0.1}
+    assert {k: v[0] for k, v in part.wanted().items()} == {k: tuple(v.shape) for k, v in ws.items()}
+    part.load(ws.__getitem__, dtype, DEV)
+    for rows in (3, 70):  # the streaming kernel and the many-row path
+        x = torch.randn(rows, 72).to(dtype)
+        ctx = make_ctx([rows], [0], [[0] * 8], 16, dtype)
+        got = part.forward(ctx, x.to(DEV))
+        ref = pl.swiglu(x, *(ws[k].to(dtype) for k in ws))
+        if dtype == torch.float32:
+            torch.testing.assert_close(got.cpu(), ref, rtol=1e-4, atol=1e-5)
+        else:
+            assert ulps_of_row_max(got.cpu(), ref).max() <= 4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("window", [0, 9])
+def test_attention_part_with_cache_across_steps(dtype, window):
+    """The mixer alone: two requests, the first step writes a portion, the second appends a portion to one and a single
+    token to the other; against plain projections + rotation + attention over the whole sequences."""
+    import math
+
+    from nanospec_amd.cache.storage import PagedView
+    from nanospec_amd.config.spec import AttentionSpec, RopeSpec
+    from nanospec_amd.parts import build
+
+    torch.manual_seed(2)
+    hidden, heads, kvh, hd, page = 80, 6, 2, 32, 8
+    spec = AttentionSpec(hidden=hidden, heads=heads, kv_heads=kvh, head_dim=hd, position=RopeSpec(rotary_dim=hd, theta=1e4),
+                         softmax_scale=1 / math.sqrt(hd), window=window)
+    part = build("mixer", spec, "a.")
+    ws = {"a.q_proj.weight": torch.randn(heads * hd, hidden) * 0.2, "a.k_proj.weight": torch.randn(kvh * hd, hidden) * 0.2,
+          "a.v_proj.weight": torch.randn(kvh * hd, hidden) * 0.2, "a.o_proj.weight": torch.randn(hidden, heads * hd) * 0.2}
+    part.load(ws.__getitem__, dtype, DEV)
+    need = part.cache_need()
+    assert (need.kv_heads, need.head_dim, need.window) == (kvh, hd, window)
+    k = torch.zeros(12, page, kvh, hd, dtype=dtype, device=DEV)
+    v = torch.zeros(12, kvh, hd, page, dtype=dtype, device=DEV)
+    cache = PagedView(0, k, v)
+    xs = [torch.randn(21, hidden).to(dtype), torch.randn(14, hidden).to(dtype)]
+    tables = [[7, 2, 9], [4, 11]]
+
+    def plain(x):
+        t = x.shape[0]
+        q = pl.linear(x, ws["a.q_proj.weight"].to(dtype)).view(t, heads, hd)
+        kk = pl.linear(x, ws["a.k_proj.weight"].to(dtype)).view(t, kvh, hd)
+        vv = pl.linear(x, ws["a.v_proj.weight"].to(dtype)).view(t, kvh, hd)
+        cos, sin = pl.rotation_tables(torch.arange(t), pl.inverse_frequencies(hd, 1e4, None))
+        q, kk = pl.rotate(q, cos, sin), pl.rotate(kk, cos, sin)
+        if window:
+            a = torch.cat([pl.causal_attention(q[i : i + 1], kk[max(0, i - window + 1) : i + 1], vv[max(0, i - window + 1) : i + 1],
+                                               first_query=min(i, window - 1)) for i in range(t)])
+        else:
+            a = pl.causal_attention(q, kk, vv)
+        return pl.linear(a.reshape(t, -1), ws["a.o_proj.weight"].to(dtype))
+
+    refs = [plain(x) for x in xs]
+    steps = [([17, 13], [0, 0]), ([4, 1], [17, 13])]
+    for lens, starts in steps:
+        ctx = make_ctx(lens, starts, tables, page, dtype)
+        x = torch.cat([xs[b][s : s + n] for b, (s, n) in enumerate(zip(starts, lens))]).to(DEV)
+        got = part.forward(ctx, x, cache, True).cpu()
+        ref = torch.cat([refs[b][s : s + n] for b, (s, n) in enumerate(zip(starts, lens))])
+        if dtype == torch.float32:
+            torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-4)
+        else:
+            assert ulps_of_row_max(got, ref).max() <= 6
+
+
+# ------------------------------------------------------------------------------------------------ a toy mixer with state
+
+
+@dataclass(frozen=True)
+class PrefixMeanSpec:
+    """out_t = W . mean(x_0 .. x_t): a mixer whose whole memory is a running sum of fixed size."""
+
+    kind: ClassVar[str] = "prefix_mean"
+    hidden: int
+
+
+class PrefixMean:
+    graph_safe = False  # plain torch operations: the engine then runs it without captured graphs
+
+    def __init__(self, spec, prefix):
+        self.spec, self.prefix, self.w = spec, prefix, None
+
+    def wanted(self):
+        return {self.prefix + "weight": ((self.spec.hidden, self.spec.hidden), "linear")}
+
+    def load(self, get, dtype, device):
+        self.w = get(self.prefix + "weight").to(device=device, dtype=torch.float32)
+
+    def cache_need(self):
+        from nanospec_amd.parts import StateNeed
+
+        return StateNeed((self.spec.hidden,), torch.float32)
+
+    def forward(self, ctx, x, cache, owns_cache=True, out=None):
+        indptr, slots = ctx.qo_indptr.tolist(), ctx.state_slots.tolist()
+        pos = ctx.positions.to(torch.float32)
+        res = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        for b, slot in enumerate(slots):
+            lo, hi = indptr[b], indptr[b + 1]
+            sums = cache.state[slot] + torch.cumsum(x[lo:hi].float(), 0)
+            cache.state[slot] = sums[-1]
+            res[lo:hi] = (sums / (pos[lo:hi, None] + 1)) @ self.w.T
+        res = res.to(x.dtype)
+        return res if out is None else out.copy_(res)
+
+
+def toy_model(dtype):
+    """Layer 0: the toy mixer.  Layer 1: attention.  Run order: 0, 1, 1 again (a cache of its own), then 1 reading the
+    cache of its first run."""
+    import math
+
+    from nanospec_amd.config.spec import (AttentionSpec, LayerCall, ModelSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec, SwiGLUSpec)
+    from nanospec_amd.parts import DecoderModel, register
+    from nanospec_amd.weights import DictSource, random_tensors
+
+    register("mixer", "prefix_mean", PrefixMean)
+    hidden, vocab = 48, 97
+    norm = RMSNormSpec(hidden, 1e-5)
+    ffn = SwiGLUSpec(hidden, 80)
+    attn = AttentionSpec(hidden, 3, 1, 16, RopeSpec(16, 1e4), 1 / math.sqrt(16))
+    layers = (PreNormBlockSpec("model.layers.0.", norm, PrefixMeanSpec(hidden), norm, ffn),
+              PreNormBlockSpec("model.layers.1.", norm, attn, norm, ffn))
+    spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers,
+                     (LayerCall(0), LayerCall(1), LayerCall(1), LayerCall(1, cache_from=1)), norm, "model.norm.weight", "lm_head.weight", True)
+    net = DecoderModel(spec)
+    assert "model.layers.0.prefix_mean.weight" in net.wanted()
+    tensors = random_tensors(net.wanted(), seed=5, skip={"lm_head.weight"})
+    tensors = {k: v * (6.0 if k.endswith("proj.weight") or k.endswith("mean.weight") else 1.0) for k, v in tensors.items()}
+    return net.load(DictSource(tensors), dtype, DEV), tensors, spec
+
+
+def toy_plain(tensors, tokens):
+    """The toy model over a whole sequence with the plain functions."""
+    w = tensors
+    x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    t = len(tokens)
+    cos, sin = pl.rotation_tables(torch.arange(t), pl.inverse_frequencies(16, 1e4, None))
+
+    def ffn(x, p):
+        h = pl.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+        return x + pl.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+
+    p0, p1 = "model.layers.0.", "model.layers.1."
+    h = pl.rms_norm(x, w[p0 + "input_layernorm.weight"], 1e-5)
+    x = ffn(x + (torch.cumsum(h, 0) / torch.arange(1, t + 1)[:, None]) @ w[p0 + "prefix_mean.weight"].T, p0)
+    first_kv = None
+    for run in range(3):
+        h = pl.rms_norm(x, w[p1 + "input_layernorm.weight"], 1e-5)
+        q = pl.rotate(pl.linear(h, w[p1 + "self_attn.q_proj.weight"]).view(t, 3, 16), cos, sin)
+        if run < 2:
+            k = pl.rotate(pl.linear(h, w[p1 + "self_attn.k_proj.weight"]).view(t, 1, 16), cos, sin)
+            v = pl.linear(h, w[p1 + "self_attn.v_proj.weight"]).view(t, 1, 16)
+            if run == 0:
+                first_kv = (k, v)
+        else:
+            k, v = first_kv  # the third run reads the cache its first run wrote
+        a = pl.causal_attention(q, k, v).reshape(t, -1)
+        x = ffn(x + pl.linear(a, w[p1 + "self_attn.o_proj.weight"]), p1)
+    return pl.rms_norm(x, w["model.norm.weight"], 1e-5) @ w["model.embed_tokens.weight"].T
+
+
+def test_toy_mixer_with_state_layer_twice_and_borrowed_cache():
+    from nanospec_amd.engine.replay import Replayer
+
+    model, tensors, spec = toy_model(torch.float32)
+    assert not model.graph_safe
+    kinds = [type(n).__name__ for n in model.cache_needs]
+    assert kinds == ["StateNeed", "PagedNeed", "PagedNeed", "NoneType"]
+    g = torch.Generator().manual_seed(0)
+    seqs = {r: torch.randint(0, 97, (n,), generator=g).tolist() for r, n in (("a", 37), ("b", 12), ("c", 29))}
+    refs = {r: toy_plain(tensors, t) for r, t in seqs.items()}
+    rep = Replayer(model, 128, page_size=4)
+    assert len(rep.storage.states) == 1 and rep.storage.k[0].shape[0] == 2  # one state tensor; two attention caches in one group
+    assert rep.storage.views[3] is rep.storage.views[1]
+
+    def step(entries, end=()):
+        out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(range(e - s))} for r, s, e in entries], list(end))
+        want = torch.cat([refs[r][s:e] for r, s, e in entries])
+        err = ((out - want).abs().amax(-1) / want.abs().amax(-1)).max()
+        assert err < 1e-4, (entries, float(err))
+
+    step([("a", 0, 10), ("b", 0, 12)], end=["b"])       # portions: the state carries over between them
+    step([("a", 10, 11)])
+    step([("a", 11, 30), ("c", 0, 2)])                  # request c gets the slot request b gave back: it must start from zero
+    step([("a", 30, 37), ("c", 2, 29)], end=["a", "c"])
+    rep.manager.check()

@@ -103,6 +103,25 @@ def test_schedules_match_plain(tiny_folders, name, dtype, schedule):
     replay(model, steps, where, ref, dtype, max_tokens, page)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding_from_the_first_token(tiny_folders, name, dtype):
+    """Two requests decoded one token at a time from position 0 to the model's last position: the first tokens of a
+    sequence (one key, then two, ...), every page edge on the way, and errors that would build up over many steps."""
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = {k: v for k, v in list(sequences(name).items())[-2:]}
+    ref = plain_logits(folder, name, dtype)
+    model = engine_model(folder, name, dtype)
+    longest = max(len(t) for t in seqs.values())
+    steps, where = [], []
+    for p in range(longest):
+        live = [r for r, t in seqs.items() if p < len(t)]
+        steps.append({"step": p, "entries": [{"id": r, "tokens": [seqs[r][p]], "want": [0]} for r in live],
+                      "end": [r for r in live if p == len(seqs[r]) - 1]})
+        where.append([(r, p) for r in live])
+    replay(model, steps, where, ref, dtype, 512, page)
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_graph_and_eager_decode_agree(tiny_folders, name):
     folder, page = tiny_folders[name], TINY[name]["page"]

@@ -1,0 +1,177 @@
+"""The scheduler's decisions, without a GPU: a stand-in for the engine reserves and commits what a step would write
+and appends a token for every request that samples.  The first two tests hold the vectors of the reference's
+tests/test_scheduler.py."""
+
+import random
+
+import pytest
+
+from nanospec_amd.cache import CacheManager, GroupSpec, PoolExhausted
+from nanospec_amd.engine.scheduler import Request, Scheduler
+from nanospec_amd.sampling import SamplingParams
+
+
+def manager(pages, page, slots=16):
+    return CacheManager([GroupSpec("all")], pages, page, slots)
+
+
+def req(i, n, max_tokens=4):
+    return Request(i, list(range(n)), SamplingParams(max_tokens=max_tokens))
+
+
+def run_step(s: Scheduler, token=1):
+    """One engine step's worth of bookkeeping.  -> the work list."""
+    work = s.next_batch()
+    for w in work:
+        w.sampled = w.samples  # as seen before any token is appended
+        s.cache.reserve(w.req.id, w.n)
+    for w in work:
+        s.cache.commit(w.req.id, w.n)
+        w.req.computed += w.n
+    for w in work:
+        if w.sampled:
+            w.req.out_tokens.append(token)
+            if len(w.req.out_tokens) >= w.req.params.max_tokens:
+                s.finish(w.req)
+    s.cache.check()
+    return work
+
+
+def ids(work):
+    return [(w.req.id, w.n) for w in work]
+
+
+def test_staggered_admission_and_decode_order():
+    """reference tests/test_scheduler.py:9-22: one admission per step; a request is prefilled in the step it is admitted
+    and decodes in the next; max_running caps."""
+    s = Scheduler(manager(64, 4), max_admit=1)
+    for i in range(3):
+        s.add(req(i, 5, max_tokens=40))
+    assert ids(run_step(s)) == [(0, 5)]
+    assert ids(run_step(s)) == [(0, 1), (1, 5)]
+    assert ids(run_step(s)) == [(0, 1), (1, 1), (2, 5)]
+    assert [s.cache.get(r.id).length for r in s.running] == [7, 6, 5]
+    s.max_running = 3
+    s.add(req(3, 5))
+    assert ids(run_step(s)) == [(0, 1), (1, 1), (2, 1)]  # the cap keeps request 3 waiting
+    assert [r.id for r in s.waiting] == [3]
+
+
+def test_admission_waits_for_pages_and_finish_frees():
+    """reference tests/test_scheduler.py:25-42: admission reserves prompt + max_tokens; strictly first come first served."""
+    m = manager(4, 4)
+    s = Scheduler(m, max_admit=8)
+    s.add(req(0, 12))  # 12 + 4 -> 4 pages
+    s.add(req(1, 6))   # 6 + 4 -> 3 pages: does not fit beside request 0
+    s.add(req(2, 1))   # 1 + 4 -> 2 pages: would fit, but may not overtake request 1
+    s._admit()
+    assert [r.id for r in s.running] == [0] and [r.id for r in s.waiting] == [1, 2]
+    s.finish(s.running[0])
+    assert m.num_free() == 4
+    s._admit()
+    assert [r.id for r in s.running] == [1]  # 3 pages spoken for, 1 left: request 2 (2 pages) waits
+    s.finish(s.running[0])
+    s._admit()
+    assert [r.id for r in s.running] == [2]
+    s.finish(s.running[0])
+    assert not s.has_work and m.num_free() == 4
+    m.check()
+
+
+def test_a_request_that_can_never_fit_is_refused_at_once():
+    s = Scheduler(manager(4, 4))
+    with pytest.raises(PoolExhausted):
+        s.add(req(0, 14, max_tokens=8))
+
+
+def test_token_budget_cuts_prompts_into_portions():
+    """Decoding requests come first with one token each; the rest of the budget goes to prompts in admission order,
+    at most prefill_chunk per request; a request samples only in the step that ends its prompt."""
+    s = Scheduler(manager(256, 4, slots=8), max_admit=8, max_step_tokens=16, prefill_chunk=10)
+    s.add(req(0, 25, max_tokens=3))
+    s.add(req(1, 7, max_tokens=3))
+    w = run_step(s)
+    assert ids(w) == [(0, 10), (1, 6)] and not any(x.sampled for x in w)
+    w = run_step(s)
+    assert ids(w) == [(0, 10), (1, 1)] and [x.sampled for x in w] == [False, True]
+    w = run_step(s)
+    assert ids(w) == [(0, 5), (1, 1)] and [x.sampled for x in w] == [True, True]  # request 1 decodes beside the last portion
+    assert ids(run_step(s)) == [(0, 1), (1, 1)]
+    assert [r.id for r in s.running] == [0]  # request 1 has its 3 tokens
+    run_step(s)
+    assert not s.has_work and s.cache.num_free() == 256
+
+
+def test_budget_smaller_than_the_decoding_requests():
+    s = Scheduler(manager(64, 4), max_admit=8, max_step_tokens=2)
+    for i in range(3):
+        s.add(req(i, 1, max_tokens=5))
+    assert ids(run_step(s)) == [(0, 1), (1, 1)]
+    assert ids(run_step(s)) == [(0, 1), (1, 1)]  # decoding requests first; request 2 waits for room in the budget
+    while s.has_work:
+        assert sum(w.n for w in run_step(s)) <= 2
+    assert s.cache.num_free() == 64
+
+
+def test_preemption_when_pages_run_out():
+    """Under "preempt" admission needs only the first portion.  When a step does not fit, the request admitted last goes
+    back to the HEAD of the queue with its output kept; later it is recomputed from prompt + output."""
+    m = manager(6, 4)
+    s = Scheduler(m, max_admit=8, on_exhaustion="preempt")
+    a, b = req(0, 8, max_tokens=12), req(1, 8, max_tokens=12)
+    s.add(a), s.add(b)
+    assert ids(run_step(s)) == [(0, 8), (1, 8)]  # 2 + 2 pages
+    for _ in range(4):
+        assert ids(run_step(s)) == [(0, 1), (1, 1)]  # 12 tokens each: 3 + 3 pages, pool full
+    w = run_step(s)  # token 13 of each needs a 4th page: only request 0 keeps running
+    assert ids(w) == [(0, 1)] and b.state == "waiting" and b.preemptions == 1 and s.waiting[0] is b
+    assert len(b.out_tokens) == 5 and b.computed == 0
+    m.check()
+    while a.state != "done":
+        run_step(s)
+    w = run_step(s)
+    assert ids(w) == [(1, 13)] and w[0].sampled  # recomputed from prompt + the 5 tokens it had
+    while s.has_work:
+        run_step(s)
+    assert len(a.out_tokens) == len(b.out_tokens) == 12 and m.num_free() == 6
+    # alone and still too long for what is left of the pool: an error, not an endless loop
+    s2 = Scheduler(manager(2, 4), on_exhaustion="preempt")
+    s2.add(Request(0, list(range(4)), SamplingParams(max_tokens=4)))
+    s2.cache.admit("someone else"), s2.cache.reserve("someone else", 1)
+    run_step(s2)
+    with pytest.raises(PoolExhausted):
+        run_step(s2)
+
+
+def test_reserve_policy_never_runs_out():
+    rng = random.Random(3)
+    m = manager(40, 4, slots=8)
+    s = Scheduler(m, max_admit=3, max_running=7, max_step_tokens=24, prefill_chunk=9)
+    reqs = [Request(i, list(range(rng.randint(1, 30))), SamplingParams(max_tokens=rng.randint(1, 20))) for i in range(40)]
+    for r in reqs:
+        s.add(r)
+    steps = 0
+    while s.has_work:
+        work = run_step(s)
+        assert work and sum(w.n for w in work) <= 24
+        steps += 1
+        assert steps < 2000
+    assert all(r.state == "done" and len(r.out_tokens) == r.params.max_tokens for r in reqs)
+    assert m.num_free() == 40 and s.preempted_total == 0
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_preempt_policy_always_finishes(seed):
+    rng = random.Random(seed)
+    m = manager(24, 4, slots=8)
+    s = Scheduler(m, max_admit=4, max_running=6, max_step_tokens=32, prefill_chunk=16, on_exhaustion="preempt")
+    reqs = [Request(i, list(range(rng.randint(1, 20))), SamplingParams(max_tokens=rng.randint(1, 30))) for i in range(25)]
+    for r in reqs:
+        s.add(r)
+    steps = 0
+    while s.has_work:
+        run_step(s)
+        steps += 1
+        assert steps < 5000
+    assert all(r.state == "done" and len(r.out_tokens) == r.params.max_tokens for r in reqs)
+    assert m.num_free() == 24 and s.preempted_total > 0
