@@ -16,7 +16,8 @@
 //                                                tokens per 8-byte load; B = P^T is exactly the
 //                                                layout S^T came out in.
 // The running maximum, the running sum and the output accumulators of a column therefore live in
-// the lanes of that column and are rescaled without any exchange.
+// the lanes of that column and are rescaled without any exchange.  Keys are walked in blocks of 32;
+// the loads of the next block are issued before the arithmetic of the current one.
 //
 // Query at position p sees keys max(0, p - window + 1) .. p.  Scores, soft-max and sums are 32-bit.
 // With splits > 1 the keys of a tile are cut into `splits` contiguous ranges of whole 32-key blocks;
@@ -28,25 +29,26 @@
 #endif
 constexpr int HD = NS_HEAD_DIM;
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
-constexpr int DT = HD / 16;         // 16-channel tiles of the output
-constexpr bool WIDE = HD % 32 == 0;  // q.k with the k=32 instruction, else with k=16
+constexpr int DT = HD / 16;           // 16-channel tiles of the output
+constexpr bool WIDE = HD % 32 == 0;   // q.k with the k=32 instruction, else with k=16
+constexpr int NQ = WIDE ? HD / 32 : HD / 16;  // q.k instructions per 16-key tile
+constexpr int TILE_INTS = 8;          // ints per tile descriptor
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
+// A tile descriptor, filled on the host: {request, first token of the tile among the request's tokens of this step,
+// row of the request's first token in the batch, tokens of the request in this step, keys after this step, 0, 0, 0}.
 struct AttnParams {
   bf16_t* out;        // [tokens, heads, HD]
-  float* part_o;      // [tokens * heads, splits, HD]   (splits > 1)
-  float* part_ml;     // [tokens * heads, splits, 2]
+  float* part_o;      // [n_tiles * (16 / hp) * heads, splits, HD]   (splits > 1)
+  float* part_ml;     // [n_tiles * (16 / hp) * heads, splits, 2]
   const bf16_t* q;    // row t at q + t * q_stride, head h at + h * HD
   const bf16_t* k_cache;
   const bf16_t* v_cache;
-  const int* tile_req;  // [n_tiles] request of the tile
-  const int* tile_t0;   // [n_tiles] first token of the tile within the request's tokens of this step
-  const int* qo_indptr;  // [requests + 1]
-  const int* kv_lens;    // [requests] keys after this step's tokens are written
+  const int* tiles;   // [n_tiles][TILE_INTS]
   const int* block_table;
   int q_stride, table_stride, n_tiles, heads, kv_heads, page_size, hp, splits, window;
   float scale_log2;  // softmax scale * log2(e)
@@ -63,6 +65,13 @@ __device__ __forceinline__ int wave_min_i(int v) {
   return v;
 }
 
+// The operands of one block of 32 keys as they come from memory.
+struct KVBlock {
+  bf16x8 kw[WIDE ? 2 * NQ : 1];  // [tile t][i]
+  s16x4 kn[WIDE ? 1 : 2 * NQ];
+  bf16x4 v[DT][2];               // [channel tile][keys 4g.. of tile 0 | of tile 1]
+};
+
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
@@ -75,13 +84,15 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const long ts = item / ny;
   const int split = (int)(ts % a.splits), tile = (int)(ts / a.splits);
   const int kvh = y / hblks, hblk = y % hblks;
-  const int b = a.tile_req[tile], t0 = a.tile_t0[tile];
-  const int q0 = a.qo_indptr[b], n = a.qo_indptr[b + 1] - q0, kv_len = a.kv_lens[b];
+  const int4 info = *reinterpret_cast<const int4*>(a.tiles + (size_t)tile * TILE_INTS);
+  const int b = info.x, t0 = info.y, q0 = info.z, n = info.w;
+  const int kv_len = a.tiles[(size_t)tile * TILE_INTS + 4];
   const int* table = a.block_table + (size_t)b * a.table_stride;
   const int ps = a.page_size;
 
   // this lane's column
-  const int ti = t0 + c / a.hp;
+  const int tt = c / a.hp;  // token of the tile
+  const int ti = t0 + tt;
   const int hin = hblk * a.hp + c % a.hp;
   const bool col_ok = ti < n && hin < G;
   const int head = kvh * G + (col_ok ? hin : 0);
@@ -89,7 +100,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const int lo = (col_ok && a.window > 0) ? max(0, pos - a.window + 1) : 0;
   const int whi = wave_max_i(pos) + 1;                    // keys [wlo, whi) are seen by some column
   const int wlo = wave_min_i(col_ok ? lo : 0x7fffffff);
-  // (a tile always holds a column; if it did not, the wave would still have to reach the counter below)
+
   int kb0 = whi > 0 ? wlo / 32 : 0, kb1 = whi > 0 ? (whi + 31) / 32 : 0;
   if (a.splits > 1) {
     const int per = (kb1 - kb0 + a.splits - 1) / a.splits;
@@ -99,17 +110,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 
   // Q^T fragments of this lane's column
   const bf16_t* qrow = a.q + (size_t)(q0 + (col_ok ? ti : 0)) * a.q_stride + head * HD;
-  bf16x8 qw[WIDE ? HD / 32 : 1];
-  s16x4 qn[WIDE ? 1 : HD / 16];
+  bf16x8 qw[WIDE ? NQ : 1];
+  s16x4 qn[WIDE ? 1 : NQ];
   if (WIDE) {
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i) {
+    for (int i = 0; i < NQ; ++i) {
       qw[i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32 + g * 8);
       if (!col_ok) qw[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < HD / 16; ++i) {
+    for (int i = 0; i < NQ; ++i) {
       qn[i] = *reinterpret_cast<const s16x4*>(qrow + i * 16 + g * 4);
       if (!col_ok) qn[i] = s16x4{0, 0, 0, 0};
     }
@@ -120,29 +131,55 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, lsum = 0.f;
   const int qlo = wlo & ~3, qhi = (whi - 1) & ~3;  // first and last 4-key group that holds a seen key
+  const size_t kv_row = (size_t)a.kv_heads * HD;   // elements per token of a K page
+  const size_t v_page = kv_row * ps;               // elements per V page
 
-  for (int kb = kb0; kb < kb1; ++kb) {
+  // Issue the loads of block kb.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
+  auto load = [&](KVBlock& blk, int kb) {
     const int key_base = kb * 32;
-    // ---- S^T = K . Q^T for two tiles of 16 keys
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);
+      const int page = table[key / ps];
+      const bf16_t* krow = a.k_cache + ((size_t)page * ps + key % ps) * kv_row + kvh * HD;
+      if (WIDE) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) blk.kw[t * NQ + i] = *reinterpret_cast<const bf16x8*>(krow + i * 32 + g * 8);
+      } else {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) blk.kn[t * NQ + i] = *reinterpret_cast<const s16x4*>(krow + i * 16 + g * 4);
+      }
+    }
+    // Slot 8 g + j of the second product holds key key_base + 4 g + j for j < 4 and key_base + 16 + 4 g + (j - 4)
+    // for j >= 4, in both operands.
+    const int k0 = min(max(key_base + g * 4, qlo), qhi);
+    const int k1 = min(max(key_base + 16 + g * 4, qlo), qhi);
+    const bf16_t* v0 = a.v_cache + (size_t)table[k0 / ps] * v_page + (size_t)kvh * HD * ps + k0 % ps;
+    const bf16_t* v1 = a.v_cache + (size_t)table[k1 / ps] * v_page + (size_t)kvh * HD * ps + k1 % ps;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const size_t ch = (size_t)(dt * 16 + c) * ps;
+      blk.v[dt][0] = *reinterpret_cast<const bf16x4*>(v0 + ch);
+      blk.v[dt][1] = *reinterpret_cast<const bf16x4*>(v1 + ch);
+    }
+  };
+
+  auto compute = [&](const KVBlock& blk, int kb) {
+    const int key_base = kb * 32;
     f32x4 s[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);  // keep the address inside held pages
-      const int page = table[key / ps];
-      const bf16_t* krow = a.k_cache + (((size_t)page * ps + key % ps) * a.kv_heads + kvh) * HD;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
       if (WIDE) {
 #pragma unroll
-        for (int i = 0; i < HD / 32; ++i)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + i * 32 + g * 8), qw[i], acc, 0, 0, 0);
+        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kw[t * NQ + i], qw[i], acc, 0, 0, 0);
       } else {
 #pragma unroll
-        for (int i = 0; i < HD / 16; ++i)
-          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s16x4*>(krow + i * 16 + g * 4), qn[i], acc, 0, 0, 0);
+        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.kn[t * NQ + i], qn[i], acc, 0, 0, 0);
       }
       s[t] = acc;
     }
-    // ---- mask, running maximum, probabilities.  s[t][j] is key key_base + 16 t + 4 g + j of column c.
+    // mask, running maximum, probabilities.  s[t][j] is key key_base + 16 t + 4 g + j of column c.
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -170,101 +207,116 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
         pf[t * 4 + j] = (bf16_t)p;
       }
     lsum = lsum * alpha + psum;
-    // ---- O^T = O^T * alpha + V^T . P^T.  Slot 8 g + j of the instruction holds key key_base + 4 g + j
-    //      for j < 4 and key_base + 16 + 4 g + (j - 4) for j >= 4, in both operands.
-    const int k0 = min(max(key_base + g * 4, qlo), qhi);
-    const int k1 = min(max(key_base + 16 + g * 4, qlo), qhi);
-    const size_t v0 = ((size_t)table[k0 / ps] * a.kv_heads + kvh) * HD * ps + k0 % ps;
-    const size_t v1 = ((size_t)table[k1 / ps] * a.kv_heads + kvh) * HD * ps + k1 % ps;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const size_t ch = (size_t)(dt * 16 + c) * ps;
-      const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(a.v_cache + v0 + ch);
-      const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(a.v_cache + v1 + ch);
+      const bf16x4 lo4 = blk.v[dt][0], hi4 = blk.v[dt][1];
       const bf16x8 vf = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
 #pragma unroll
       for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
     }
+  };
+
+  KVBlock ba, bb;
+  int kb = kb0;
+  if (kb < kb1) load(ba, kb);
+  while (kb + 1 < kb1) {
+    load(bb, kb + 1);
+    compute(ba, kb);
+    if (kb + 2 < kb1) load(ba, kb + 2);
+    compute(bb, kb + 1);
+    kb += 2;
   }
+  if (kb < kb1) compute(ba, kb);
 
   lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
+  if (!col_ok) return;
   // o[dt][j] is channel 16 dt + 4 g + j of column c
-  const size_t col = (size_t)(q0 + (col_ok ? ti : 0)) * a.heads + head;
   if (a.splits == 1) {
-    if (!col_ok) return;
+    const size_t col = (size_t)(q0 + ti) * a.heads + head;
     const float inv = 1.f / lsum;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       bf16x4 r = {(bf16_t)(o[dt][0] * inv), (bf16_t)(o[dt][1] * inv), (bf16_t)(o[dt][2] * inv), (bf16_t)(o[dt][3] * inv)};
       *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
     }
-  } else if (col_ok) {
-    float* po = a.part_o + (col * a.splits + split) * HD;
+  } else {
+    const size_t pcol = ((size_t)tile * (16 / a.hp) + tt) * a.heads + head;
+    float* po = a.part_o + (pcol * a.splits + split) * HD;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
     if (g == 0) {
-      a.part_ml[(col * a.splits + split) * 2] = m;
-      a.part_ml[(col * a.splits + split) * 2 + 1] = lsum;
+      a.part_ml[(pcol * a.splits + split) * 2] = m;
+      a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum;
     }
   }
 }
 
 // Joining the key ranges: out[col] = sum_s o_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*), m* = max_s m_s.
-// One wave per (tile, head) and token of the tile; lane s first holds range s (at most 64 ranges), so the maxima
-// and weights are formed by wave reductions, then the lanes split the channels and add the ranges in order.
+// One wave per (tile, token of the tile, head); lane s first holds range s (at most 64 ranges), so the maxima and
+// weights are formed by wave reductions, then the lanes split the channels and add the ranges in order.  The ranges'
+// results are addressed by tile, so nothing here waits for the tile descriptor except the final store.
 __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
-                                                         const float* __restrict__ part_ml,
-                                                         const int* __restrict__ tile_req, const int* __restrict__ tile_t0,
-                                                         const int* __restrict__ qo_indptr, int heads, int hp, int splits) {
-  const int b = tile_req[blockIdx.x], t0 = tile_t0[blockIdx.x], head = blockIdx.y;
-  const int q0 = qo_indptr[b], n = qo_indptr[b + 1] - q0;
-  const int t1 = min(n, t0 + 16 / hp);
+                                                         const float* __restrict__ part_ml, const int* __restrict__ tiles,
+                                                         int heads, int hp, int splits) {
+  const int tile = blockIdx.x, head = blockIdx.y, tt = blockIdx.z;
   const int lane = threadIdx.x;
-  for (int ti = t0; ti < t1; ++ti) {
-    const size_t col = (size_t)(q0 + ti) * heads + head;
-    const float* ml = part_ml + col * splits * 2;
-    float ms = -INFINITY, ls = 0.f;
-    if (lane < splits) {
-      ms = ml[lane * 2];
-      ls = ml[lane * 2 + 1];
-    }
-    float mstar = ms;
+  const size_t pcol = ((size_t)tile * (16 / hp) + tt) * heads + head;
+  const float* ml = part_ml + pcol * splits * 2;
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < splits) {
+    ms = ml[lane * 2];
+    ls = ml[lane * 2 + 1];
+  }
+  constexpr int PER = (HD + 63) / 64;
+  const float* po = part_o + pcol * splits * HD;
+  const int4 info = *reinterpret_cast<const int4*>(tiles + (size_t)tile * TILE_INTS);
+  const int ti = info.y + tt;
+  if (ti >= info.w) return;  // the tile holds fewer tokens
+  float mstar = ms;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, o, 64));
-    const float wgt = ms == -INFINITY ? 0.f : exp2f(ms - mstar);
-    float l = ls * wgt;
+  for (int o = 32; o > 0; o >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, o, 64));
+  const float wgt = ms == -INFINITY ? 0.f : exp2f(ms - mstar);
+  float l = ls * wgt;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
-    const float inv = 1.f / l;
-    for (int d = lane; d < HD; d += 64) {
-      float acc = 0.f;
-      const float* po = part_o + col * splits * HD + d;
-      for (int s = 0; s < splits; ++s) acc += po[(size_t)s * HD] * __shfl(wgt, s, 64);
-      out[col * HD + d] = (bf16_t)(acc * inv);
+  for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+  const float inv = 1.f / l;
+  float acc[PER];
+#pragma unroll
+  for (int p = 0; p < PER; ++p) acc[p] = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ws = __shfl(wgt, s, 64);
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int d = lane + p * 64;
+      if (d < HD) acc[p] += po[(size_t)s * HD + d] * ws;
     }
+  }
+  const size_t col = (size_t)(info.z + ti) * heads + head;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int d = lane + p * 64;
+    if (d < HD) out[col * HD + d] = (bf16_t)(acc[p] * inv);
   }
 }
 
 extern "C" int ns_attn_mfma_head_dim() { return HD; }
 
-// Workspace, when splits > 1: part_o holds tokens*heads*splits*HD floats, part_ml tokens*heads*splits*2.
+// Workspace, when splits > 1: part_o holds n_tiles*(16/hp)*heads*splits*HD floats, part_ml n_tiles*(16/hp)*heads*splits*2.
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
-                            const void* v_cache, const int* tile_req, const int* tile_t0, const int* qo_indptr,
-                            const int* kv_lens, const int* block_table, int table_stride, int n_tiles, int n_tokens,
+                            const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale,
                             hipStream_t stream) {
-  if (n_tiles <= 0 || n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || (page_size & 3) ||
-      window < 0 || splits < 1 || (q_stride & 7))
+  if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || (page_size & 3) || window < 0 ||
+      splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
     return NS_ERR_BAD_ARG;
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
-  if (splits > 64) return NS_ERR_BAD_ARG;
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
   AttnParams a;
   a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
   a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
-  a.tile_req = tile_req; a.tile_t0 = tile_t0; a.qo_indptr = qo_indptr; a.kv_lens = kv_lens; a.block_table = block_table;
+  a.tiles = tiles; a.block_table = block_table;
   a.q_stride = q_stride; a.table_stride = table_stride; a.n_tiles = n_tiles; a.heads = heads; a.kv_heads = kv_heads;
   a.page_size = page_size; a.hp = hp; a.splits = splits; a.window = window;
   a.scale_log2 = scale * 1.4426950408889634f;
@@ -276,7 +328,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const int st = ns_launch_status();
   if (st != NS_OK || splits == 1) return st;
   if (heads > 65535) return NS_ERR_BAD_ARG;
-  attn_reduce_kernel<<<dim3(n_tiles, heads), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml, tile_req,
-                                                             tile_t0, qo_indptr, heads, hp, splits);
+  attn_reduce_kernel<<<dim3(n_tiles, heads, 16 / hp), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml,
+                                                                      tiles, heads, hp, splits);
   return ns_launch_status();
 }

@@ -7,8 +7,9 @@ kv_indptr / kv_indices / kv_last_page_len / positions / slots):
     token_ids[N] positions[N] token_req[N]        per token; token_req = index of its request in the batch
     qo_indptr[B+1] kv_lens[B] state_slots[B]      per request; kv_lens counts the keys after this step
     want_rows[R]                                  token rows whose logits are wanted
-    chunk tiles (tile_req, tile_t0)[Tc]           requests with more than one token, 16 tokens per tile
-    decode tiles (tile_req, tile_t0)[Td]          requests with exactly one token
+    chunk tiles [Tc, 8]                           requests with more than one token, 16 tokens per tile; a tile is
+    decode tiles [Td, 8]                          (request, first token, first row, tokens, keys, 0, 0, 0); decode
+                                                  tiles are the requests with exactly one token
     block_table[g][B, P]                          page of positions [i*page, (i+1)*page), -1 if released
 Slots are not materialised: the kernels compute page and offset from the position and the block table.
 """
@@ -21,6 +22,7 @@ import numpy as np
 import torch
 
 CHUNK_TILE = 16  # tokens per attention tile of a prompt portion
+TILE_INTS = 8  # a tile descriptor: request, first token, row of the request's first token, tokens, keys, 0, 0, 0
 
 
 def _pad4(n: int) -> int:
@@ -36,8 +38,8 @@ class BatchLayout:
         off = 0
         self.fields = {}
         for name, size in (("token_ids", n_tokens), ("positions", n_tokens), ("token_req", n_tokens), ("qo_indptr", n_reqs + 1),
-                           ("kv_lens", n_reqs), ("state_slots", n_reqs), ("want_rows", n_want), ("ctile_req", n_chunk_tiles),
-                           ("ctile_t0", n_chunk_tiles), ("dtile_req", n_decode_tiles), ("dtile_t0", n_decode_tiles)):
+                           ("kv_lens", n_reqs), ("state_slots", n_reqs), ("want_rows", n_want),
+                           ("ctiles", TILE_INTS * n_chunk_tiles), ("dtiles", TILE_INTS * n_decode_tiles)):
             self.fields[name] = (off, size)
             off += _pad4(max(size, 1))
         self.table_off = []
@@ -49,8 +51,7 @@ class BatchLayout:
 
 @dataclass
 class AttentionPlan:
-    tile_req: torch.Tensor
-    tile_t0: torch.Tensor
+    tiles: torch.Tensor  # int32 [n_tiles, 8]
     hp: int
     splits: int
     workspace: tuple | None
@@ -73,8 +74,8 @@ class StepContext:
         self.token_ids, self.positions, self.token_req = view("token_ids"), view("positions"), view("token_req")
         self.qo_indptr, self.kv_lens, self.state_slots = view("qo_indptr"), view("kv_lens"), view("state_slots")
         self.want_rows = view("want_rows")
-        self._ctiles = (view("ctile_req"), view("ctile_t0"))
-        self._dtiles = (view("dtile_req"), view("dtile_t0"))
+        self._ctiles = view("ctiles").view(-1, TILE_INTS)
+        self._dtiles = view("dtiles").view(-1, TILE_INTS)
         self.block_tables = [dev_buf[o : o + layout.B * layout.P].view(layout.B, layout.P) for o in layout.table_off]
 
     def attention_plans(self, group: int, kv_heads: int, head_dim: int) -> list[AttentionPlan]:
@@ -84,7 +85,7 @@ class StepContext:
         plans = []  # made afresh per call: the workspace lives in the caller's arena scope
         lay = self.layout
         if lay.Tc:
-            plans.append(AttentionPlan(self._ctiles[0], self._ctiles[1], 1, 1, None))
+            plans.append(AttentionPlan(self._ctiles, 1, 1, None))
         if lay.Td:
             hp = 1
             while hp < min(group, 16):
@@ -95,9 +96,9 @@ class StepContext:
                 splits = max(1, min(splits, -(-self.max_kv_len // 128)))
             ws = None
             if splits > 1:
-                cols = lay.N * kv_heads * group
+                cols = lay.Td * (16 // hp) * kv_heads * group
                 ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
-            plans.append(AttentionPlan(self._dtiles[0], self._dtiles[1], hp, splits, ws))
+            plans.append(AttentionPlan(self._dtiles, hp, splits, ws))
         return plans
 
 
@@ -124,20 +125,15 @@ def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, s
     put("state_slots", np.asarray(slots, dtype=np.int32))
     if layout.R:
         put("want_rows", np.asarray(want_rows, dtype=np.int32))
-    ct_req, ct_t0, dt_req = [], [], []
-    for b, n in enumerate(lens):
-        if n == 1:
-            dt_req.append(b)
-        else:
-            for t0 in range(0, n, CHUNK_TILE):
-                ct_req.append(b)
-                ct_t0.append(t0)
-    if layout.Tc:
-        put("ctile_req", np.asarray(ct_req, dtype=np.int32))
-        put("ctile_t0", np.asarray(ct_t0, dtype=np.int32))
+    kv = starts_a + lens_a
     if layout.Td:
-        put("dtile_req", np.asarray(dt_req, dtype=np.int32))
-        put("dtile_t0", np.zeros(len(dt_req), dtype=np.int32))
+        req = np.nonzero(lens_a == 1)[0].astype(np.int32)
+        d = np.zeros((len(req), TILE_INTS), dtype=np.int32)
+        d[:, 0], d[:, 2], d[:, 3], d[:, 4] = req, indptr[req], 1, kv[req]
+        put("dtiles", d.reshape(-1))
+    if layout.Tc:
+        rows = [(b, t0, indptr[b], n, kv[b], 0, 0, 0) for b, n in enumerate(lens) if n != 1 for t0 in range(0, n, CHUNK_TILE)]
+        put("ctiles", np.asarray(rows, dtype=np.int32).reshape(-1))
     for g, off in enumerate(layout.table_off):
         host[off : off + B * layout.P] = tables[g].reshape(-1)
 

@@ -79,9 +79,8 @@ class Attention:
         if ops.mfma_attention_takes(x.dtype, s.head_dim, page):
             group = s.heads // s.kv_heads
             for plan in ctx.attention_plans(group, s.kv_heads, s.head_dim):
-                ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tile_req, plan.tile_t0, ctx.qo_indptr, ctx.kv_lens, table,
-                                   s.heads, s.kv_heads, s.head_dim, s.softmax_scale, window=s.window, hp=plan.hp,
-                                   splits=plan.splits, workspace=plan.workspace)
+                ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim,
+                                   s.softmax_scale, window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace)
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)

@@ -265,25 +265,26 @@ def test_attention_generic(dtype, case, heads, kvh, hd, page):
 
 def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None):
     n = sum(lens)
-    B = len(lens)
-    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
-    kv_lens = torch.tensor([s + l for s, l in zip(starts, lens)], dtype=torch.int32, device=DEV)
+    indptr = [0]
+    for l in lens:
+        indptr.append(indptr[-1] + l)
     out = torch.zeros(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     group = heads // kvh
-    ct = [(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16)]
-    dt = [(b, 0) for b, l in enumerate(lens) if l == 1]
+    tile = lambda b, t0: [b, t0, indptr[b], lens[b], starts[b] + lens[b], 0, 0, 0]
+    ct = [tile(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16)]
+    dt = [tile(b, 0) for b, l in enumerate(lens) if l == 1]
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
     if ct:
-        ops.attention_mfma(q, out, k, v, i32([c[0] for c in ct]), i32([c[1] for c in ct]), indptr, kv_lens, table.to(DEV), heads, kvh,
-                           hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1)
+        ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1)
     if dt:
         hp = 1
         while hp < min(group, 16):
             hp *= 2
         splits = force_splits or 3
-        ws = (torch.empty(n * heads * splits * hd, dtype=torch.float32, device=DEV), torch.empty(n * heads * splits * 2, dtype=torch.float32, device=DEV))
-        ops.attention_mfma(q, out, k, v, i32([d[0] for d in dt]), i32([0] * len(dt)), indptr, kv_lens, table.to(DEV), heads, kvh, hd,
-                           1 / math.sqrt(hd), window=window, hp=hp, splits=splits, workspace=ws if splits > 1 else None)
+        cols = len(dt) * (16 // hp) * heads
+        ws = (torch.empty(cols * splits * hd, dtype=torch.float32, device=DEV), torch.empty(cols * splits * 2, dtype=torch.float32, device=DEV))
+        ops.attention_mfma(q, out, k, v, i32(dt), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=hp,
+                           splits=splits, workspace=ws if splits > 1 else None)
     return out
 
 
