@@ -39,7 +39,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-// A tile descriptor, filled on the host: {request, first token of the tile among the request's tokens of this step,
+// A tile descriptor, filled on the host: {request, first token of the tile among the request's tokens of this step
+// (tiles of one request follow each other every 16 qt / hp tokens),
 // row of the request's first token in the batch, tokens of the request in this step, keys after this step, 0, 0, 0}.
 struct AttnParams {
   bf16_t* out;        // [tokens, heads, HD]
@@ -50,7 +51,7 @@ struct AttnParams {
   const bf16_t* v_cache;
   const int* tiles;   // [n_tiles][TILE_INTS]
   const int* block_table;
-  int q_stride, table_stride, n_tiles, heads, kv_heads, page_size, hp, splits, window;
+  int q_stride, table_stride, n_tiles, heads, kv_heads, page_shift, hp, splits, window;
   float scale_log2;  // softmax scale * log2(e)
 };
 
@@ -72,6 +73,9 @@ struct KVBlock {
   bf16x4 v[DT][2];               // [channel tile][keys 4g.. of tile 0 | of tile 1]
 };
 
+// QT: tiles of 16 columns per wave (2 only with hp == 1: 32 tokens of one head share every load of K and V).
+// PREFETCH: the loads of the next key block are issued before the arithmetic of the current one.
+template <int QT, bool PREFETCH>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
@@ -88,18 +92,26 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const int b = info.x, t0 = info.y, q0 = info.z, n = info.w;
   const int kv_len = a.tiles[(size_t)tile * TILE_INTS + 4];
   const int* table = a.block_table + (size_t)b * a.table_stride;
-  const int ps = a.page_size;
+  const int psh = a.page_shift, pmask = (1 << a.page_shift) - 1;
 
-  // this lane's column
-  const int tt = c / a.hp;  // token of the tile
-  const int ti = t0 + tt;
+  // this lane's columns: column c of sub-tile u
+  const int tt0 = c / a.hp;  // token of the tile (sub-tile 0)
   const int hin = hblk * a.hp + c % a.hp;
-  const bool col_ok = ti < n && hin < G;
-  const int head = kvh * G + (col_ok ? hin : 0);
-  const int pos = col_ok ? kv_len - n + ti : -1;
-  const int lo = (col_ok && a.window > 0) ? max(0, pos - a.window + 1) : 0;
-  const int whi = wave_max_i(pos) + 1;                    // keys [wlo, whi) are seen by some column
-  const int wlo = wave_min_i(col_ok ? lo : 0x7fffffff);
+  const int head = kvh * G + (hin < G ? hin : 0);
+  bool col_ok[QT];
+  int pos[QT], lo[QT];
+  int whi = 0, wlo = 0x7fffffff, full_hi = 0x7fffffff, full_lo = 0;
+#pragma unroll
+  for (int u = 0; u < QT; ++u) {
+    const int ti = t0 + u * (16 / a.hp) + tt0;
+    col_ok[u] = ti < n && hin < G;
+    pos[u] = col_ok[u] ? kv_len - n + ti : -1;
+    lo[u] = (col_ok[u] && a.window > 0) ? max(0, pos[u] - a.window + 1) : 0;
+    whi = max(whi, wave_max_i(pos[u]) + 1);                       // keys [wlo, whi) are seen by some column
+    wlo = min(wlo, wave_min_i(col_ok[u] ? lo[u] : 0x7fffffff));
+    full_hi = min(full_hi, wave_min_i(col_ok[u] ? pos[u] : 0x7fffffff));  // keys <= full_hi are seen by every column
+    full_lo = max(full_lo, wave_max_i(lo[u]));                             // ... if they are >= full_lo
+  }
 
   int kb0 = whi > 0 ? wlo / 32 : 0, kb1 = whi > 0 ? (whi + 31) / 32 : 0;
   if (a.splits > 1) {
@@ -108,31 +120,42 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     kb1 = min(kb1, kb0 + per);
   }
 
-  // Q^T fragments of this lane's column
-  const bf16_t* qrow = a.q + (size_t)(q0 + (col_ok ? ti : 0)) * a.q_stride + head * HD;
-  bf16x8 qw[WIDE ? NQ : 1];
-  s16x4 qn[WIDE ? 1 : NQ];
-  if (WIDE) {
+  // Q^T fragments of this lane's columns
+  bf16x8 qw[QT][WIDE ? NQ : 1];
+  s16x4 qn[QT][WIDE ? 1 : NQ];
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      qw[i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32 + g * 8);
-      if (!col_ok) qw[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-  } else {
+  for (int u = 0; u < QT; ++u) {
+    const int ti = t0 + u * (16 / a.hp) + tt0;
+    const bf16_t* qrow = a.q + (size_t)(q0 + (col_ok[u] ? ti : 0)) * a.q_stride + head * HD;
+    if (WIDE) {
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      qn[i] = *reinterpret_cast<const s16x4*>(qrow + i * 16 + g * 4);
-      if (!col_ok) qn[i] = s16x4{0, 0, 0, 0};
+      for (int i = 0; i < NQ; ++i) {
+        qw[u][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32 + g * 8);
+        if (!col_ok[u]) qw[u][i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) {
+        qn[u][i] = *reinterpret_cast<const s16x4*>(qrow + i * 16 + g * 4);
+        if (!col_ok[u]) qn[u][i] = s16x4{0, 0, 0, 0};
+      }
     }
   }
 
-  f32x4 o[DT];
+  f32x4 o[QT][DT];
+  float m[QT], lsum[QT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, lsum = 0.f;
+  for (int u = 0; u < QT; ++u) {
+    m[u] = -INFINITY;
+    lsum[u] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[u][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
   const int qlo = wlo & ~3, qhi = (whi - 1) & ~3;  // first and last 4-key group that holds a seen key
   const size_t kv_row = (size_t)a.kv_heads * HD;   // elements per token of a K page
-  const size_t v_page = kv_row * ps;               // elements per V page
+  const bf16_t* kbase = a.k_cache + (size_t)kvh * HD + (WIDE ? g * 8 : g * 4);
+  const bf16_t* vbase = a.v_cache + (((size_t)kvh * HD + c) << psh);
+  const size_t v_step = (size_t)16 << psh;  // elements between channel tiles of a V page
 
   // Issue the loads of block kb.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
   auto load = [&](KVBlock& blk, int kb) {
@@ -140,115 +163,148 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);
-      const int page = table[key / ps];
-      const bf16_t* krow = a.k_cache + ((size_t)page * ps + key % ps) * kv_row + kvh * HD;
+      const int page = table[key >> psh];
+      const bf16_t* krow = kbase + (((size_t)page << psh) + (key & pmask)) * kv_row;
       if (WIDE) {
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) blk.kw[t * NQ + i] = *reinterpret_cast<const bf16x8*>(krow + i * 32 + g * 8);
+        for (int i = 0; i < NQ; ++i) blk.kw[t * NQ + i] = *reinterpret_cast<const bf16x8*>(krow + i * 32);
       } else {
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) blk.kn[t * NQ + i] = *reinterpret_cast<const s16x4*>(krow + i * 16 + g * 4);
+        for (int i = 0; i < NQ; ++i) blk.kn[t * NQ + i] = *reinterpret_cast<const s16x4*>(krow + i * 16);
       }
     }
     // Slot 8 g + j of the second product holds key key_base + 4 g + j for j < 4 and key_base + 16 + 4 g + (j - 4)
     // for j >= 4, in both operands.
     const int k0 = min(max(key_base + g * 4, qlo), qhi);
     const int k1 = min(max(key_base + 16 + g * 4, qlo), qhi);
-    const bf16_t* v0 = a.v_cache + (size_t)table[k0 / ps] * v_page + (size_t)kvh * HD * ps + k0 % ps;
-    const bf16_t* v1 = a.v_cache + (size_t)table[k1 / ps] * v_page + (size_t)kvh * HD * ps + k1 % ps;
+    const bf16_t* v0 = vbase + (((size_t)table[k0 >> psh] * kv_row) << psh) + (k0 & pmask);
+    const bf16_t* v1 = vbase + (((size_t)table[k1 >> psh] * kv_row) << psh) + (k1 & pmask);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const size_t ch = (size_t)(dt * 16 + c) * ps;
-      blk.v[dt][0] = *reinterpret_cast<const bf16x4*>(v0 + ch);
-      blk.v[dt][1] = *reinterpret_cast<const bf16x4*>(v1 + ch);
+      blk.v[dt][0] = *reinterpret_cast<const bf16x4*>(v0 + dt * v_step);
+      blk.v[dt][1] = *reinterpret_cast<const bf16x4*>(v1 + dt * v_step);
     }
   };
 
   auto compute = [&](const KVBlock& blk, int kb) {
     const int key_base = kb * 32;
-    f32x4 s[2];
+    // every key of the block is seen by every column: no masks needed (uniform over the wave)
+    const bool full = key_base + 31 <= full_hi && key_base >= full_lo;
+    bf16x8 pf[QT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      if (WIDE) {
+    for (int u = 0; u < QT; ++u) {
+      f32x4 s[2];
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kw[t * NQ + i], qw[i], acc, 0, 0, 0);
+      for (int t = 0; t < 2; ++t) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (WIDE) {
+#pragma unroll
+          for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kw[t * NQ + i], qw[u][i], acc, 0, 0, 0);
+        } else {
+#pragma unroll
+          for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.kn[t * NQ + i], qn[u][i], acc, 0, 0, 0);
+        }
+        s[t] = acc;
+      }
+      // s[t][j] is key key_base + 16 t + 4 g + j of column c
+      float mx = -INFINITY;
+      if (full) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            s[t][j] *= a.scale_log2;
+            mx = fmaxf(mx, s[t][j]);
+          }
       } else {
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.kn[t * NQ + i], qn[i], acc, 0, 0, 0);
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int key = key_base + t * 16 + g * 4 + j;
+            const float v = (key >= lo[u] && key <= pos[u]) ? s[t][j] * a.scale_log2 : -INFINITY;
+            s[t][j] = v;
+            mx = fmaxf(mx, v);
+          }
       }
-      s[t] = acc;
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[u], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const bool moved = m_new != m[u];
+      const float alpha = exp2f(m[u] - m_safe);
+      m[u] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float p = exp2f(s[t][j] - m_safe);
+          psum += p;
+          pf[u][t * 4 + j] = (bf16_t)p;
+        }
+      if (__any(moved)) {  // the maximum settles early in long rows; rescaling is skipped from then on
+        lsum[u] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[u][dt][j] *= alpha;
+      }
+      lsum[u] += psum;
     }
-    // mask, running maximum, probabilities.  s[t][j] is key key_base + 16 t + 4 g + j of column c.
-    float mx = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int key = key_base + t * 16 + g * 4 + j;
-        const float v = (key >= lo && key <= pos) ? s[t][j] * a.scale_log2 : -INFINITY;
-        s[t][j] = v;
-        mx = fmaxf(mx, v);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f(m - m_safe);
-    m = m_new;
-    float psum = 0.f;
-    bf16x8 pf;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float p = exp2f(s[t][j] - m_safe);
-        psum += p;
-        pf[t * 4 + j] = (bf16_t)p;
-      }
-    lsum = lsum * alpha + psum;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       const bf16x4 lo4 = blk.v[dt][0], hi4 = blk.v[dt][1];
       const bf16x8 vf = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+      for (int u = 0; u < QT; ++u) o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
     }
   };
 
-  KVBlock ba, bb;
-  int kb = kb0;
-  if (kb < kb1) load(ba, kb);
-  while (kb + 1 < kb1) {
-    load(bb, kb + 1);
-    compute(ba, kb);
-    if (kb + 2 < kb1) load(ba, kb + 2);
-    compute(bb, kb + 1);
-    kb += 2;
-  }
-  if (kb < kb1) compute(ba, kb);
-
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
-  if (!col_ok) return;
-  // o[dt][j] is channel 16 dt + 4 g + j of column c
-  if (a.splits == 1) {
-    const size_t col = (size_t)(q0 + ti) * a.heads + head;
-    const float inv = 1.f / lsum;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      bf16x4 r = {(bf16_t)(o[dt][0] * inv), (bf16_t)(o[dt][1] * inv), (bf16_t)(o[dt][2] * inv), (bf16_t)(o[dt][3] * inv)};
-      *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
+  if (PREFETCH) {
+    KVBlock ba, bb;
+    int kb = kb0;
+    if (kb < kb1) load(ba, kb);
+    while (kb + 1 < kb1) {
+      load(bb, kb + 1);
+      compute(ba, kb);
+      if (kb + 2 < kb1) load(ba, kb + 2);
+      compute(bb, kb + 1);
+      kb += 2;
     }
+    if (kb < kb1) compute(ba, kb);
   } else {
-    const size_t pcol = ((size_t)tile * (16 / a.hp) + tt) * a.heads + head;
-    float* po = a.part_o + (pcol * a.splits + split) * HD;
+    KVBlock ba;
+    for (int kb = kb0; kb < kb1; ++kb) {
+      load(ba, kb);
+      compute(ba, kb);
+    }
+  }
+
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
-    if (g == 0) {
-      a.part_ml[(pcol * a.splits + split) * 2] = m;
-      a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum;
+  for (int u = 0; u < QT; ++u) {
+    lsum[u] += __shfl_xor(lsum[u], 16, 64);
+    lsum[u] += __shfl_xor(lsum[u], 32, 64);
+    if (!col_ok[u]) continue;
+    const int tt = u * (16 / a.hp) + tt0;
+    // o[u][dt][j] is channel 16 dt + 4 g + j of column c
+    if (a.splits == 1) {
+      const size_t col = (size_t)(q0 + t0 + tt) * a.heads + head;
+      const float inv = 1.f / lsum[u];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        bf16x4 r = {(bf16_t)(o[u][dt][0] * inv), (bf16_t)(o[u][dt][1] * inv), (bf16_t)(o[u][dt][2] * inv), (bf16_t)(o[u][dt][3] * inv)};
+        *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
+      }
+    } else {
+      const size_t pcol = ((size_t)tile * (16 / a.hp) + tt) * a.heads + head;
+      float* po = a.part_o + (pcol * a.splits + split) * HD;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[u][dt];
+      if (g == 0) {
+        a.part_ml[(pcol * a.splits + split) * 2] = m[u];
+        a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum[u];
+      }
     }
   }
 }
@@ -285,12 +341,20 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ ou
   float acc[PER];
 #pragma unroll
   for (int p = 0; p < PER; ++p) acc[p] = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ws = __shfl(wgt, s, 64);
+  for (int s0 = 0; s0 < splits; s0 += 8) {  // eight ranges' loads in flight at a time
+    float v[8][PER];
 #pragma unroll
-    for (int p = 0; p < PER; ++p) {
-      const int d = lane + p * 64;
-      if (d < HD) acc[p] += po[(size_t)s * HD + d] * ws;
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int p = 0; p < PER; ++p) {
+        const int d = lane + p * 64;
+        v[i][p] = (s0 + i < splits && d < HD) ? po[(size_t)(s0 + i) * HD + d] : 0.f;
+      }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float ws = __shfl(wgt, (s0 + i) & 63, 64);
+#pragma unroll
+      for (int p = 0; p < PER; ++p) acc[p] += v[i][p] * ws;
     }
   }
   const size_t col = (size_t)(info.z + ti) * heads + head;
@@ -306,25 +370,29 @@ extern "C" int ns_attn_mfma_head_dim() { return HD; }
 // Workspace, when splits > 1: part_o holds n_tiles*(16/hp)*heads*splits*HD floats, part_ml n_tiles*(16/hp)*heads*splits*2.
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
-                            int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale,
+                            int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
                             hipStream_t stream) {
-  if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || (page_size & 3) || window < 0 ||
+  if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size < 4 || (page_size & (page_size - 1)) || window < 0 ||
       splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
     return NS_ERR_BAD_ARG;
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
+  if (qt != 1 && !(qt == 2 && hp == 1 && splits == 1)) return NS_ERR_BAD_ARG;
   AttnParams a;
   a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
   a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
   a.tiles = tiles; a.block_table = block_table;
   a.q_stride = q_stride; a.table_stride = table_stride; a.n_tiles = n_tiles; a.heads = heads; a.kv_heads = kv_heads;
-  a.page_size = page_size; a.hp = hp; a.splits = splits; a.window = window;
+  a.page_shift = __builtin_ctz(page_size); a.hp = hp; a.splits = splits; a.window = window;
   a.scale_log2 = scale * 1.4426950408889634f;
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);
   const long blocks = (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
-  attn_mfma_kernel<<<(unsigned)blocks, 256, 0, stream>>>(a);
+  if (qt == 2)
+    attn_mfma_kernel<2, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
+  else
+    attn_mfma_kernel<1, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
   const int st = ns_launch_status();
   if (st != NS_OK || splits == 1) return st;
   if (heads > 65535) return NS_ERR_BAD_ARG;

@@ -7,7 +7,7 @@ kv_indptr / kv_indices / kv_last_page_len / positions / slots):
     token_ids[N] positions[N] token_req[N]        per token; token_req = index of its request in the batch
     qo_indptr[B+1] kv_lens[B] state_slots[B]      per request; kv_lens counts the keys after this step
     want_rows[R]                                  token rows whose logits are wanted
-    chunk tiles [Tc, 8]                           requests with more than one token, 16 tokens per tile; a tile is
+    chunk tiles [Tc, 8]                           requests with more than one token, 32 tokens per tile; a tile is
     decode tiles [Td, 8]                          (request, first token, first row, tokens, keys, 0, 0, 0); decode
                                                   tiles are the requests with exactly one token
     block_table[g][B, P]                          page of positions [i*page, (i+1)*page), -1 if released
@@ -21,7 +21,7 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
-CHUNK_TILE = 16  # tokens per attention tile of a prompt portion
+CHUNK_TILE = 32  # tokens per attention tile of a prompt portion (two 16-column tiles per wave)
 TILE_INTS = 8  # a tile descriptor: request, first token, row of the request's first token, tokens, keys, 0, 0, 0
 
 
@@ -55,6 +55,7 @@ class AttentionPlan:
     hp: int
     splits: int
     workspace: tuple | None
+    qt: int = 1
 
 
 class StepContext:
@@ -80,12 +81,12 @@ class StepContext:
 
     def attention_plans(self, group: int, kv_heads: int, head_dim: int) -> list[AttentionPlan]:
         """How the matrix-core attention kernel is launched for a mixer with ``group`` query heads per
-        key/value head: prompt portions as 16-token tiles of one head; decode rows with all heads of a
+        key/value head: prompt portions as 32-token tiles of one head; decode rows with all heads of a
         group in one tile and the keys cut into ranges so that the launch fills the GPU."""
         plans = []  # made afresh per call: the workspace lives in the caller's arena scope
         lay = self.layout
         if lay.Tc:
-            plans.append(AttentionPlan(self._ctiles, 1, 1, None))
+            plans.append(AttentionPlan(self._ctiles, 1, 1, None, qt=CHUNK_TILE // 16))
         if lay.Td:
             hp = 1
             while hp < min(group, 16):

@@ -290,7 +290,7 @@ def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_tabl
 
 
 def mfma_attention_takes(dtype, head_dim: int, page_size: int) -> bool:
-    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and page_size % 4 == 0
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and page_size >= 4 and page_size & (page_size - 1) == 0
 
 
 TILE_INTS = 8  # ints per attention tile descriptor: request, first token, first row, tokens, keys, 0, 0, 0
@@ -298,22 +298,24 @@ TILE_INTS = 8  # ints per attention tile descriptor: request, first token, first
 
 def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_heads: int, head_dim: int, scale: float,
                    window: int = 0, hp: int = 1, splits: int = 1,
-                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1) -> torch.Tensor:
     """bfloat16 attention on the matrix cores for the tiles described in ``tiles`` (int32 [n_tiles, 8]: request, first
     token of the tile among the request's tokens of this step, row of the request's first token in ``q``, tokens of the
     request in this step, keys after this step, three zeros).  ``hp`` heads of a group times 16/hp tokens make a tile;
-    ``splits`` > 1 cuts the keys of every tile into that many ranges (at most 64) and needs ``workspace`` =
-    (part_o, part_ml) float32 tensors."""
+    with ``qt`` = 2 (only with hp = 1 and no splits) a tile is 32 tokens.  ``splits`` > 1 cuts the keys of every tile
+    into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
     if not mfma_attention_takes(q.dtype, head_dim, page):
         raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
-                            f"multiples of 4; got {q.dtype}, head size {head_dim}, page {page}")
+                            f"powers of two from 4; got {q.dtype}, head size {head_dim}, page {page}")
     _gpu(tiles, block_table)
     _i32(tiles, "tiles"), _i32(block_table, "block_table")
     if tiles.dim() != 2 or tiles.shape[1] != TILE_INTS or tiles.data_ptr() % 16:
         raise KernelRefused(f"attention_mfma: tiles must be int32 [n_tiles, {TILE_INTS}], 16-byte aligned")
     if hp not in (1, 2, 4, 8, 16):
         raise KernelRefused("attention_mfma: hp is a power of two up to 16")
+    if qt != 1 and not (qt == 2 and hp == 1 and splits == 1):
+        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1 and no splits")
     n_tiles = tiles.shape[0]
     po = pm = None
     if splits > 1:
@@ -326,7 +328,7 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     lib = build.attn(head_dim)
     _check(lib.ns_attn_mfma(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tiles),
                             _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads),
-                            c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), _stream()), "attention_mfma")
+                            c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), _stream()), "attention_mfma")
     return out
 
 

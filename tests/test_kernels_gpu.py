@@ -263,7 +263,7 @@ def test_attention_generic(dtype, case, heads, kvh, hd, page):
         assert ulps_of_row_max(out.cpu(), ref).max() <= 4  # the reference's bound, tests/test_backends.py:71
 
 
-def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None):
+def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2):
     n = sum(lens)
     indptr = [0]
     for l in lens:
@@ -271,11 +271,11 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
     out = torch.zeros(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     group = heads // kvh
     tile = lambda b, t0: [b, t0, indptr[b], lens[b], starts[b] + lens[b], 0, 0, 0]
-    ct = [tile(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16)]
+    ct = [tile(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16 * qt)]
     dt = [tile(b, 0) for b, l in enumerate(lens) if l == 1]
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
     if ct:
-        ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1)
+        ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1, qt=qt)
     if dt:
         hp = 1
         while hp < min(group, 16):
@@ -302,10 +302,10 @@ def test_attention_mfma(case, heads, kvh, hd, page):
     n = sum(lens)
     q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
-    for splits in (1, 3, 7):
-        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits)
+    for splits, qt in ((1, 2), (3, 1), (7, 2), (33, 1)):
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt)
         u = ulps_of_row_max(out.cpu(), ref).max()
-        assert u <= 4, f"{case} splits={splits}: {u:.2f} ulps"
+        assert u <= 4, f"{case} splits={splits} qt={qt}: {u:.2f} ulps"
 
 
 @pytest.mark.parametrize("kernel", ["generic", "mfma"])
