@@ -1,5 +1,5 @@
 // Soft-max attention over the paged bfloat16 cache on the matrix cores, for prefill portions and for
-// decode, compiled for one head size (NS_HEAD_DIM, a multiple of 16 up to 256).
+// decode, compiled for one head size (NS_HEAD_DIM, a multiple of 16 up to 256) and one page size (NS_PAGE_SIZE).
 //
 // One wave owns one tile of 16 "columns".  A column is a (query token, query head) pair of one
 // request and one key/value head: hp consecutive heads of the group times 16/hp consecutive tokens.
@@ -24,10 +24,12 @@
 // each range writes its un-normalised output, maximum and sum, and a second small kernel joins them.
 #include "common.h"
 
-#ifndef NS_HEAD_DIM
-#error "compile with -DNS_HEAD_DIM=<multiple of 16>"
+#if !defined(NS_HEAD_DIM) || !defined(NS_PAGE_SIZE)
+#error "compile with -DNS_HEAD_DIM=<multiple of 16> -DNS_PAGE_SIZE=<power of two from 4>"
 #endif
 constexpr int HD = NS_HEAD_DIM;
+constexpr int PS = NS_PAGE_SIZE;  // tokens per cache page: a constant, so that page arithmetic is shifts and offsets are immediates
+static_assert(PS >= 4 && (PS & (PS - 1)) == 0, "page size must be a power of two from 4");
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
 constexpr int DT = HD / 16;           // 16-channel tiles of the output
 constexpr bool WIDE = HD % 32 == 0;   // q.k with the k=32 instruction, else with k=16
@@ -51,9 +53,12 @@ struct AttnParams {
   const bf16_t* v_cache;
   const int* tiles;   // [n_tiles][TILE_INTS]
   const int* block_table;
-  int q_stride, table_stride, n_tiles, heads, kv_heads, page_shift, hp, splits, window;
+  int q_stride, table_stride, n_tiles, heads, kv_heads, hp, splits, window;
   float scale_log2;  // softmax scale * log2(e)
 };
+
+// 2^x by the hardware instruction alone: arguments here are <= 0, and results below the normal range may flush to 0.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ int wave_max_i(int v) {
 #pragma unroll
@@ -86,13 +91,14 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   if (item >= (long)a.n_tiles * a.splits * ny) return;
   const int y = (int)(item % ny);
   const long ts = item / ny;
-  const int split = (int)(ts % a.splits), tile = (int)(ts / a.splits);
+  // tiles are listed in the order of the tokens; the last ones see the most keys, so they start first
+  const int split = (int)(ts % a.splits), tile = a.n_tiles - 1 - (int)(ts / a.splits);
   const int kvh = y / hblks, hblk = y % hblks;
   const int4 info = *reinterpret_cast<const int4*>(a.tiles + (size_t)tile * TILE_INTS);
   const int b = info.x, t0 = info.y, q0 = info.z, n = info.w;
   const int kv_len = a.tiles[(size_t)tile * TILE_INTS + 4];
   const int* table = a.block_table + (size_t)b * a.table_stride;
-  const int psh = a.page_shift, pmask = (1 << a.page_shift) - 1;
+  constexpr int psh = __builtin_ctz(PS), pmask = PS - 1;
 
   // this lane's columns: column c of sub-tile u
   const int tt0 = c / a.hp;  // token of the tile (sub-tile 0)
@@ -155,7 +161,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const size_t kv_row = (size_t)a.kv_heads * HD;   // elements per token of a K page
   const bf16_t* kbase = a.k_cache + (size_t)kvh * HD + (WIDE ? g * 8 : g * 4);
   const bf16_t* vbase = a.v_cache + (((size_t)kvh * HD + c) << psh);
-  const size_t v_step = (size_t)16 << psh;  // elements between channel tiles of a V page
+  constexpr size_t v_step = (size_t)16 * PS;  // elements between channel tiles of a V page
 
   // Issue the loads of block kb.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
   auto load = [&](KVBlock& blk, int kb) {
@@ -208,21 +214,19 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       }
       // s[t][j] is key key_base + 16 t + 4 g + j of column c
       float mx = -INFINITY;
+      // m[u] is the running maximum of the raw scores (the scale is positive); p = 2^((s - m) scale log2 e)
       if (full) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            s[t][j] *= a.scale_log2;
-            mx = fmaxf(mx, s[t][j]);
-          }
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[t][j]);
       } else {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int key = key_base + t * 16 + g * 4 + j;
-            const float v = (key >= lo[u] && key <= pos[u]) ? s[t][j] * a.scale_log2 : -INFINITY;
+            const float v = (key >= lo[u] && key <= pos[u]) ? s[t][j] : -INFINITY;
             s[t][j] = v;
             mx = fmaxf(mx, v);
           }
@@ -232,14 +236,15 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       const float m_new = fmaxf(m[u], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const bool moved = m_new != m[u];
-      const float alpha = exp2f(m[u] - m_safe);
+      const float alpha = fast_exp2((m[u] - m_safe) * a.scale_log2);
+      const float shift = -m_safe * a.scale_log2;
       m[u] = m_new;
       float psum = 0.f;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = exp2f(s[t][j] - m_safe);
+          const float p = fast_exp2(fmaf(s[t][j], a.scale_log2, shift));
           psum += p;
           pf[u][t * 4 + j] = (bf16_t)p;
         }
@@ -302,7 +307,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[u][dt];
       if (g == 0) {
-        a.part_ml[(pcol * a.splits + split) * 2] = m[u];
+        a.part_ml[(pcol * a.splits + split) * 2] = m[u] * a.scale_log2;  // in the exponent's units
         a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum[u];
       }
     }
@@ -366,16 +371,18 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ ou
 }
 
 extern "C" int ns_attn_mfma_head_dim() { return HD; }
+extern "C" int ns_attn_mfma_page_size() { return PS; }
 
 // Workspace, when splits > 1: part_o holds n_tiles*(16/hp)*heads*splits*HD floats, part_ml n_tiles*(16/hp)*heads*splits*2.
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
                             hipStream_t stream) {
-  if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size < 4 || (page_size & (page_size - 1)) || window < 0 ||
+  if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size != PS || window < 0 ||
       splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
     return NS_ERR_BAD_ARG;
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
+  if (!(scale > 0.f)) return NS_ERR_BAD_ARG;  // maxima are tracked on unscaled scores
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
   if (qt != 1 && !(qt == 2 && hp == 1 && splits == 1)) return NS_ERR_BAD_ARG;
   AttnParams a;
@@ -383,7 +390,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
   a.tiles = tiles; a.block_table = block_table;
   a.q_stride = q_stride; a.table_stride = table_stride; a.n_tiles = n_tiles; a.heads = heads; a.kv_heads = kv_heads;
-  a.page_shift = __builtin_ctz(page_size); a.hp = hp; a.splits = splits; a.window = window;
+  a.hp = hp; a.splits = splits; a.window = window;
   a.scale_log2 = scale * 1.4426950408889634f;
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);

@@ -4,7 +4,8 @@ Libraries are built with ``hipcc`` into ``csrc/_build`` inside the package (or, 
 writable, into a per-user folder under the temporary directory) and loaded with ``ctypes``.  A
 library is rebuilt when its sources or flags change.  The core library holds every kernel whose
 sizes are run-time arguments; the matrix-core attention kernels keep their accumulators in
-registers and are therefore compiled once per head size, on first use of that size.
+registers and address pages with constant arithmetic; they are therefore compiled once per (head size,
+page size), on first use of that pair.
 
 There is no fallback: if ``hipcc`` is missing or a source does not compile, loading raises.
 """
@@ -110,17 +111,21 @@ def core() -> ctypes.CDLL:
     return load_library("ns_core", CORE_SOURCES)
 
 
-def attn_name(head_dim: int) -> str:
-    return f"ns_attn_hd{head_dim}"
+def attn_name(head_dim: int, page_size: int) -> str:
+    return f"ns_attn_hd{head_dim}_p{page_size}"
 
 
-def attn(head_dim: int) -> ctypes.CDLL:
-    """The matrix-core attention kernels for one head size."""
-    return load_library(attn_name(head_dim), ATTN_SOURCES, [f"-DNS_HEAD_DIM={head_dim}"])
+def _attn_defines(head_dim: int, page_size: int) -> list[str]:
+    return [f"-DNS_HEAD_DIM={head_dim}", f"-DNS_PAGE_SIZE={page_size}"]
 
 
-def build_all(head_dims=(16, 32, 64, 128), force: bool = True) -> None:
-    """Compile the core library and the attention library of each given head size."""
+def attn(head_dim: int, page_size: int) -> ctypes.CDLL:
+    """The matrix-core attention kernels for one head size and one page size."""
+    return load_library(attn_name(head_dim, page_size), ATTN_SOURCES, _attn_defines(head_dim, page_size))
+
+
+def build_all(attn_variants=((16, 4), (32, 8), (64, 16), (128, 16)), force: bool = True) -> None:
+    """Compile the core library and the attention library of each given (head size, page size)."""
     compile_library("ns_core", CORE_SOURCES, force=force)
-    for hd in head_dims:
-        compile_library(attn_name(hd), ATTN_SOURCES, [f"-DNS_HEAD_DIM={hd}"], force=force)
+    for hd, page in attn_variants:
+        compile_library(attn_name(hd, page), ATTN_SOURCES, _attn_defines(hd, page), force=force)
