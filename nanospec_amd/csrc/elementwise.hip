@@ -289,3 +289,16 @@ extern "C" int ns_fill_u32(void* p, uint32_t value, size_t n_words, hipStream_t 
   fill_u32_kernel<<<blocks, 256, 0, stream>>>((uint32_t*)p, value, n_words);
   return ns_launch_status();
 }
+
+// dst[dst_idx[i]] = src[src_idx[i]]: token ids sampled by one step become the input ids of the next without a trip
+// to the host.
+__global__ void scatter_i32_kernel(int* __restrict__ dst, const int* __restrict__ dst_idx, const int* __restrict__ src,
+                                   const int* __restrict__ src_idx, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[dst_idx[i]] = src[src_idx[i]];
+}
+extern "C" int ns_scatter_i32(int* dst, const int* dst_idx, const int* src, const int* src_idx, int n, hipStream_t stream) {
+  if (n <= 0) return NS_OK;
+  scatter_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, dst_idx, src, src_idx, n);
+  return ns_launch_status();
+}

@@ -15,7 +15,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage, plan_groups
 from ..sampling.params import SamplingParams, TokenInfo
-from ..sampling.sampler import sample_rows
+from ..sampling.sampler import SampleStage, launch_sample
 from .runner import ModelRunner, StepEntry
 from .scheduler import Request, Scheduler, Work
 
@@ -34,6 +34,7 @@ class EngineConfig:
     prefill_chunk: int | None = None  # longest portion of one prompt in a step
     on_exhaustion: str = "reserve"  # "reserve" | "preempt": see engine/scheduler.py
     max_seq_len: int | None = None  # longest request (sizes the block tables); None = the whole pool
+    lookahead: bool = True  # enqueue the next decode step before waiting for this one's tokens
 
 
 class Engine:
@@ -62,6 +63,8 @@ class Engine:
         self.prof: dict[str, list[float]] = {}
         self._events: list[tuple[str, torch.cuda.Event]] = []
         self.steps = 0
+        self._ahead: dict | None = None  # a decode step that was enqueued ahead of its turn
+        self._stage = SampleStage(config.head_chunk)
 
     # ------------------------------------------------------------------ profiling (reference: engine/engine.py:83-95)
 
@@ -99,43 +102,110 @@ class Engine:
 
     # ------------------------------------------------------------------ one step
 
+    @property
+    def has_work(self) -> bool:
+        return self.sched.has_work
+
     def step(self) -> list[Request]:
-        """Admit, run one batch, sample, emit.  -> the requests that finished in this step."""
-        work = self.sched.next_batch()
-        if not work:
-            return []
+        """Admit, run one batch, sample, emit.  -> the requests that finished in this step.
+
+        With ``lookahead`` (the default) a decode-only step whose requests go on is followed at once by the launch of
+        the next step, whose input ids are taken on the GPU from this step's samples; only then does the host wait for
+        this step's tokens.  The host's work between two steps is hidden behind the GPU's.  A request that turns out to
+        have stopped on an end-of-sequence token has then already been given one more step, whose result is dropped."""
+        launched, self._ahead = self._ahead, None
+        if launched is None:
+            work = self.sched.next_batch()
+            if not work:
+                return []
+            launched = self._launch(work, None)
+        if self._may_look_ahead(launched):
+            self._ahead = self._launch_ahead(launched)
+        return self._harvest(launched)
+
+    def _launch(self, work: list[Work], token_src) -> dict:
+        """Enqueue one step and its sampling.  ``token_src``: the launched step whose samples are this step's input ids."""
         self.steps += 1
         self._mark("start")
-        entries = [StepEntry(w.req.id, [w.req.token(i) for i in range(w.start, w.start + w.n)], [w.n - 1] if w.samples else [])
-                   for w in work]
-        logits = self.runner.step(entries)
+        device_tokens = None
+        if token_src is None:
+            entries = [StepEntry(w.req.id, [w.req.token(i) for i in range(w.start, w.start + w.n)], [w.n - 1] if w.samples else [])
+                       for w in work]
+        else:
+            row_of = {id(w.req): i for i, w in enumerate(token_src["sampling"])}
+            entries = [StepEntry(w.req.id, [0], [0]) for w in work]
+            device_tokens = (token_src["sampled"][0][0], [(j, row_of[id(w.req)]) for j, w in enumerate(work)])
+        samples = [w.samples for w in work] if token_src is None else [True] * len(work)
+        logits = self.runner.step(entries, device_tokens)
         self._mark("forward")
         for w in work:
             w.req.computed += w.n
-        sampling = [w for w in work if w.samples]
-        finished: list[Request] = []
+        sampling = [w for w, smp in zip(work, samples) if smp]
+        sampled, staged, kept = [], [], []
         if sampling:
-            infos: list[TokenInfo] = []
             with torch.cuda.stream(self.runner.stream):
                 for s in range(0, len(sampling), self.config.head_chunk):
                     chunk = sampling[s : s + self.config.head_chunk]
                     # one uniform per request and step from its own generator (reference: engine/engine.py:283)
                     u = [float(torch.rand(1, generator=w.req.gen)) for w in chunk]
                     rows = logits[s : s + len(chunk)]
-                    infos.extend(sample_rows(rows, [w.req.params for w in chunk], u))
+                    sampled.append(launch_sample(rows, [w.req.params for w in chunk], u, self._stage))
+                    staged.append(self._stage.stage(sampled[-1]))
                     if self.config.record_logits:
-                        cpu = rows.cpu()
-                        for i, w in enumerate(chunk):
-                            w.req.step_logits.append(cpu[i].clone())
+                        kept.append(rows.cpu())
             self._mark("sample")
-            for w, info in zip(sampling, infos):
-                req = w.req
-                req.out_tokens.append(info.token)
-                if req.params.logprobs:
-                    req.logprobs.append(info)
-                # the stopping token is kept; the last token is never fed back (reference: engine/engine.py:155-163)
-                if info.token in self.eos or len(req.out_tokens) >= req.params.max_tokens:
-                    self.sched.finish(req)
-                    finished.append(req)
+        return {"work": work, "sampling": sampling, "sampled": sampled, "staged": staged, "logits": kept,
+                "graph": self.runner.last_used_graph}
+
+    def _harvest(self, launched: dict) -> list[Request]:
+        """Wait for a launched step's tokens, emit them, finish what is finished."""
+        finished: list[Request] = []
+        infos: list[TokenInfo] = []
+        for chunk in launched["staged"]:  # waits for this step's samples only, not for a step enqueued after it
+            infos.extend(self._stage.read(chunk))
+        row = 0
+        for w, info in zip(launched["sampling"], infos):
+            req = w.req
+            if req.state == "done":  # stopped on an end-of-sequence token while this step was already under way
+                row += 1
+                continue
+            if launched["logits"]:
+                cpu = launched["logits"][row // self.config.head_chunk]
+                req.step_logits.append(cpu[row % self.config.head_chunk].clone())
+            row += 1
+            req.out_tokens.append(info.token)
+            if req.params.logprobs:
+                req.logprobs.append(info)
+            # the stopping token is kept; the last token is never fed back (reference: engine/engine.py:155-163)
+            if info.token in self.eos or len(req.out_tokens) >= req.params.max_tokens:
+                self.sched.finish(req)
+                finished.append(req)
         self._flush_prof()
         return finished
+
+    def _may_look_ahead(self, launched: dict) -> bool:
+        c = self.config
+        if not c.lookahead or c.record_logits or c.profile or not launched["graph"] or self.sched.waiting:
+            return False
+        work = launched["work"]
+        if len(work) != len(self.sched.running) or len(launched["sampling"]) != len(work):
+            return False
+        if c.max_step_tokens is not None and len(work) > c.max_step_tokens:
+            return False
+        # whoever reaches max_tokens with the token now being sampled stops; the others go on (unless that token ends them)
+        return any(len(w.req.out_tokens) + 1 < w.req.params.max_tokens for w in work)
+
+    def _launch_ahead(self, launched: dict) -> dict | None:
+        from ..cache.pages import PoolExhausted
+
+        work = [Work(w.req, w.req.computed, 1) for w in launched["work"] if len(w.req.out_tokens) + 1 < w.req.params.max_tokens]
+        need = [0] * len(self.cache.groups)
+        for w in work:
+            for g, n in enumerate(self.cache.pages_missing(w.req.id, 1)):
+                need[g] += n
+        if any(n > self.cache.num_free(g) for g, n in enumerate(need)):
+            return None  # let the scheduler decide who is preempted
+        try:
+            return self._launch(work, launched)
+        except PoolExhausted:
+            return None

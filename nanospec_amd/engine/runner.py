@@ -41,7 +41,7 @@ class _DecodeGraph:
     def __init__(self, runner: "ModelRunner", size: int) -> None:
         self.size = size
         n_groups = len(runner.manager.groups)
-        self.layout = BatchLayout(size, size, size, 0, size, n_groups, runner.table_width)
+        self.layout = BatchLayout(size, size, size, 0, size, n_groups, runner.table_width, n_patch=size)
         dev = runner.device
         self.dev_buf = torch.zeros(self.layout.total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
@@ -108,9 +108,13 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ the step
 
-    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: list[StepEntry], device_tokens=None) -> torch.Tensor | None:
         """Run one batch.  -> float32 logits [number of wanted places, vocab] in the order of the entries
-        and of their ``want`` lists, or None if nothing is wanted."""
+        and of their ``want`` lists, or None if nothing is wanted.  Nothing here waits for the GPU.
+
+        ``device_tokens`` = (int32 tensor on the GPU, [(entry index, row of the tensor), ...]): the first token id of
+        those entries is taken from the tensor when the step runs (the id in ``tokens`` is a placeholder), so that a
+        step can be enqueued before the step that samples its input has finished."""
         if not entries:
             return None
         vocab = self.model.spec.vocab_size
@@ -140,10 +144,10 @@ class ModelRunner:
             self._staged.synchronize()  # the last batch has left the pinned staging buffers
         with torch.cuda.stream(self.stream):
             if self.use_graphs and all(n == 1 for n in lens) and n_want and self._bucket(len(entries)) is not None:
-                logits = self._step_graph(entries, rcs, starts)
+                logits = self._step_graph(entries, rcs, starts, device_tokens)
                 self.last_used_graph = True
             else:
-                logits = self._step_eager(entries, rcs, starts, lens, n_want)
+                logits = self._step_eager(entries, rcs, starts, lens, n_want, device_tokens)
                 self.last_used_graph = False
         caller.wait_stream(self.stream)  # the caller's stream sees the logits
         for e, rc in zip(entries, rcs):
@@ -164,12 +168,26 @@ class ModelRunner:
         for e in entries:
             mgr.reserve(e.req_id, len(e.tokens))
 
-    def _step_eager(self, entries, rcs, starts, lens, n_want):
+    @staticmethod
+    def _put_patch(host, layout, dst_rows, src_rows) -> None:
+        off, size = layout.fields["patch_dst"]
+        host[off : off + len(dst_rows)] = dst_rows
+        off, size = layout.fields["patch_src"]
+        host[off : off + len(src_rows)] = src_rows
+
+    @staticmethod
+    def _apply_patch(dev, layout, src, n) -> None:
+        f = layout.fields
+        ids = dev[f["token_ids"][0] : f["token_ids"][0] + f["token_ids"][1]]
+        ops.scatter_i32(ids, dev[f["patch_dst"][0] : f["patch_dst"][0] + n], src, dev[f["patch_src"][0] : f["patch_src"][0] + n])
+
+    def _step_eager(self, entries, rcs, starts, lens, n_want, device_tokens=None):
         n_tokens = sum(lens)
         tc, td = count_tiles(lens)
         max_kv = max(s + n for s, n in zip(starts, lens))
         width = max(1, -(-max_kv // self.page_size))
-        layout = BatchLayout(n_tokens, len(entries), n_want, tc, td, len(self._tables), width)
+        n_patch = len(device_tokens[1]) if device_tokens else 0
+        layout = BatchLayout(n_tokens, len(entries), n_want, tc, td, len(self._tables), width, n_patch)
         if layout.total > self._host.numel():
             size = 1 << (layout.total - 1).bit_length()
             self._host = torch.zeros(size, dtype=torch.int32).pin_memory()
@@ -182,9 +200,14 @@ class ModelRunner:
             base += n
         tables = [t[slots, :width] for t in self._tables]
         fill_batch(self._host.numpy(), layout, token_ids, starts, lens, slots, want_rows, tables)
+        if n_patch:
+            first_row = np.concatenate(([0], np.cumsum(lens)[:-1]))
+            self._put_patch(self._host.numpy(), layout, [int(first_row[e]) for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
         self._dev[: layout.total].copy_(self._host[: layout.total], non_blocking=True)
         self._staged = torch.cuda.Event()
         self._staged.record(self.stream)
+        if n_patch:
+            self._apply_patch(self._dev, layout, device_tokens[0], n_patch)
         self.arena.reset()
         ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv)
         resid, delta = self.model.forward_hidden(ctx, self.storage.views)
@@ -204,7 +227,7 @@ class ModelRunner:
             self._mirror(self.manager.get(PAD_REQUEST))
             self._pad_ready = True
 
-    def _fill_graph(self, g: _DecodeGraph, entries, rcs, starts) -> None:
+    def _fill_graph(self, g: _DecodeGraph, entries, rcs, starts, device_tokens=None) -> None:
         """Real rows first, then pad rows that read and write the reserved pad page at position 0
         (reference: engine/graphs.py:115-167)."""
         pad = self.manager.get(PAD_REQUEST)
@@ -214,9 +237,13 @@ class ModelRunner:
         st = list(starts) + [0] * n_pad
         tables = [t[slots, :] for t in self._tables]
         fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables)
+        if device_tokens:
+            self._put_patch(g.host_np, g.layout, [e for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
         g.dev_buf.copy_(g.host, non_blocking=True)
         self._staged = torch.cuda.Event()
         self._staged.record(self.stream)
+        if device_tokens:
+            self._apply_patch(g.dev_buf, g.layout, device_tokens[0], len(device_tokens[1]))
 
     def _capture(self, size: int) -> _DecodeGraph:
         g = _DecodeGraph(self, size)
@@ -239,7 +266,7 @@ class ModelRunner:
         self._graphs[size] = g
         return g
 
-    def _step_graph(self, entries, rcs, starts):
+    def _step_graph(self, entries, rcs, starts, device_tokens=None):
         self._ensure_pad()
         size = self._bucket(len(entries))
         g = self._graphs.get(size) or self._capture(size)
@@ -247,7 +274,7 @@ class ModelRunner:
         if -(-max_kv // self.page_size) > self.table_width:
             raise ValueError("a request is longer than the block tables of the captured graphs")
         self._check_positions(max_kv - 1)
-        self._fill_graph(g, entries, rcs, starts)
+        self._fill_graph(g, entries, rcs, starts, device_tokens)
         g.graph.launch()
         rows = [i for i, e in enumerate(entries) if e.want]
         if len(rows) == len(entries):

@@ -147,6 +147,16 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
     _check(build.core().ns_fill_u32(_ptr(t), c_uint32(value), c_size_t(nbytes // 4), _stream()), "fill_u32")
 
 
+def scatter_i32(dst: torch.Tensor, dst_idx: torch.Tensor, src: torch.Tensor, src_idx: torch.Tensor) -> None:
+    """dst[dst_idx[i]] = src[src_idx[i]] for int32 tensors on the GPU (indices are trusted: the caller built them)."""
+    _gpu(dst, dst_idx, src, src_idx)
+    for name, t in (("dst", dst), ("dst_idx", dst_idx), ("src", src), ("src_idx", src_idx)):
+        _i32(t, name)
+    if dst_idx.numel() != src_idx.numel():
+        raise KernelRefused("scatter_i32: one source index per destination index")
+    _check(build.core().ns_scatter_i32(_ptr(dst), _ptr(dst_idx), _ptr(src), _ptr(src_idx), c_int(dst_idx.numel()), _stream()), "scatter_i32")
+
+
 # ------------------------------------------------------------------------------------------------ matrix products
 
 

@@ -13,16 +13,81 @@ from ..kernels import ops
 from .params import SamplingParams, TokenInfo
 
 
-def sample_rows(logits: torch.Tensor, params: list[SamplingParams], uniforms: list[float]) -> list[TokenInfo]:
-    """logits float32 [rows, vocab] on the GPU -> one TokenInfo per row.  Synchronises once."""
+def launch_sample(logits: torch.Tensor, params: list[SamplingParams], uniforms: list[float], stage: "SampleStage | None" = None):
+    """logits float32 [rows, vocab] on the GPU -> (token int32, raw log-probability, processed log-probability) tensors
+    on the GPU.  Waits for nothing: with a ``stage`` the options travel through pinned memory (a copy from ordinary host
+    memory would wait for everything enqueued before it)."""
     dev = logits.device
     rows = logits.shape[0]
     if rows != len(params) or rows != len(uniforms):
         raise ValueError("one set of sampling options and one uniform number per row are wanted")
-    host = torch.tensor([[p.temperature, p.top_p, u] for p, u in zip(params, uniforms)], dtype=torch.float32).t().contiguous()
-    f = host.to(dev, non_blocking=True)
+    # (contiguous buffers only: a copy between host and GPU of a strided view goes through a temporary and waits)
+    host = stage.options(rows) if stage is not None else torch.empty((4, rows), dtype=torch.int32)
+    fl = host[:3].view(torch.float32)
+    fl[0] = torch.tensor([p.temperature for p in params], dtype=torch.float32)
+    fl[1] = torch.tensor([p.top_p for p in params], dtype=torch.float32)
+    fl[2] = torch.tensor(uniforms, dtype=torch.float32)
+    host[3] = torch.tensor([p.top_k for p in params], dtype=torch.int32)
+    d = torch.empty((4, rows), dtype=torch.int32, device=dev)
+    d.copy_(host, non_blocking=True)
+    if stage is not None:
+        stage.sent(host)
+    f = d[:3].view(torch.float32)
     filtered = any(p.top_k > 0 or p.top_p < 1.0 for p in params)
-    top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(dev) if filtered else None
-    tok, lp, slp = ops.sample(logits, f[0], f[2], top_k=top_k, top_p=f[1] if filtered else None)
-    packed = torch.stack([tok.to(torch.float32), lp, slp]).tolist()  # the step's one synchronisation
-    return [TokenInfo(int(packed[0][i]), packed[1][i], packed[2][i]) for i in range(rows)]
+    return ops.sample(logits, f[0], f[2], top_k=d[3] if filtered else None, top_p=f[1] if filtered else None)
+
+
+class SampleStage:
+    """Pinned host buffers that sampled rows are copied into as soon as they exist, each copy followed by an event, so
+    that reading one step's tokens waits for that step only and not for whatever was enqueued after it.  A buffer is
+    taken by ``stage`` and given back by ``read``."""
+
+    def __init__(self, rows: int) -> None:
+        self.rows = rows
+        self.free: list[torch.Tensor] = []
+        self._options: list[tuple[torch.Tensor, torch.cuda.Event | None]] = []  # pinned [4, rows] int32 and their copies' events
+
+    def options(self, rows: int) -> torch.Tensor:
+        """A pinned buffer for the options of ``rows`` rows whose last copy to the GPU has finished."""
+        if rows <= self.rows:
+            for i, (buf, ev) in enumerate(self._options):
+                if ev is None or ev.query():
+                    del self._options[i]
+                    return buf[: 4 * rows].view(4, rows)
+        return torch.empty(4 * max(rows, self.rows), dtype=torch.int32).pin_memory()[: 4 * rows].view(4, rows)
+
+    def sent(self, view: torch.Tensor) -> None:
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream())
+        base = view._base if view._base is not None else view
+        if base.numel() == 4 * self.rows:
+            self._options.append((base, ev))
+
+    def stage(self, sampled):
+        tok, lp, slp = sampled
+        n = tok.numel()
+        host = self.free.pop() if self.free else torch.empty(3 * max(self.rows, n), dtype=torch.float32).pin_memory()
+        host[: 3 * n].copy_(torch.stack([tok.to(torch.float32), lp, slp]).view(-1), non_blocking=True)
+        done = torch.cuda.Event()
+        done.record(torch.cuda.current_stream(tok.device))
+        return host, n, done
+
+    def read(self, staged) -> list[TokenInfo]:
+        """The step's one wait for the GPU (reference: the single ``.tolist()`` of engine/engine.py:403)."""
+        host, n, done = staged
+        done.synchronize()
+        packed = host[: 3 * n].view(3, n).tolist()
+        if host.numel() == 3 * self.rows:
+            self.free.append(host)
+        return [TokenInfo(int(packed[0][i]), packed[1][i], packed[2][i]) for i in range(n)]
+
+
+def read_sample(sampled) -> list[TokenInfo]:
+    tok, lp, slp = sampled
+    packed = torch.stack([tok.to(torch.float32), lp, slp]).tolist()
+    return [TokenInfo(int(packed[0][i]), packed[1][i], packed[2][i]) for i in range(tok.numel())]
+
+
+def sample_rows(logits: torch.Tensor, params: list[SamplingParams], uniforms: list[float]) -> list[TokenInfo]:
+    """logits float32 [rows, vocab] on the GPU -> one TokenInfo per row.  Synchronises once."""
+    return read_sample(launch_sample(logits, params, uniforms))

@@ -218,6 +218,30 @@ def test_eos_stops_and_is_kept(tiny_folders, tmp_path):
     assert out == toks[: first + 1]
 
 
+def test_lookahead_changes_nothing_but_the_timing(tiny_folders, tmp_path):
+    """Decode steps enqueued ahead of their turn take their input ids from the GPU; tokens, stops on end-of-sequence
+    (found one step late, the extra step dropped) and the state of the pool must be those of step-by-step running."""
+    import shutil
+
+    from nanospec_amd import SamplingParams, load_model
+
+    folder = tmp_path / "B_eos"
+    shutil.copytree(tiny_folders["B"], folder)
+    ref = plain_greedy(tiny_folders["B"], "B", torch.float32)
+    stops = sorted({ref[1][0][7], ref[3][0][11]})
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": stops}))
+    model = load_model(folder, dtype="float32")
+    prompts = prompts_of("B")
+    params = [SamplingParams(max_tokens=NEW["B"] - 3 * i, temperature=0.0 if i % 2 else 0.9, seed=i) for i in range(len(prompts))]
+    outs = {}
+    for ahead in (False, True):
+        reqs, _, eng = run_engine(model, prompts, params, num_blocks=96, block_size=8, lookahead=ahead)
+        outs[ahead] = [r.out_tokens for r in reqs]
+        assert all(len(r.out_tokens) <= p.max_tokens for r, p in zip(reqs, params))
+    assert outs[True] == outs[False]
+    assert any(o[-1] in stops and len(o) < p.max_tokens for o, p in zip(outs[True], params)), "no request stopped on an end token"
+
+
 def test_refuses_what_it_cannot_run(tiny_folders):
     from nanospec_amd import Engine, EngineConfig, SamplingParams
     from nanospec_amd.cache import PoolExhausted
