@@ -19,6 +19,22 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 #define EPI_STORE 0
 #define EPI_SILU_MUL 1
+#define EPI_ROPE_KV 2
+
+// What the q/k/v epilogue needs: the rows of the stacked [q; k; v] matrix were permuted at load time so that a
+// workgroup's 16 rows are, for the rotary part of a q or k head, 8 channels j and their partners j + rot/2, and
+// otherwise 16 consecutive channels.  The epilogue rotates (angle = position * inv_freq[j], 32-bit), writes q into
+// the attention input, k into its K page slot and v into the transposed V page
+// (reference: model/llama.py:175-183; kv/cache.py:23-26).
+struct RopeKvParams {
+  const int* positions;    // [M]
+  const int* token_req;    // [M]
+  const int* block_table;  // [requests, table_stride]
+  const float* inv_freq;   // [rot / 2]
+  bf16_t* k_cache;         // [pages, page, kv_heads, hd]
+  bf16_t* v_cache;         // [pages, kv_heads, hd, page]
+  int table_stride, heads, kv_heads, hd, rot, page_size, write_kv;
+};
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
@@ -146,7 +162,7 @@ template <int MT, int WAVES, int EPI, typename OutT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict__ out, const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ wt,
                                                                  const bf16_t* __restrict__ wt2, int M, int N, int K,
-                                                                 int x_stride, int out_stride) {
+                                                                 int x_stride, int out_stride, RopeKvParams rk) {
   constexpr int NACC = EPI == EPI_SILU_MUL ? 2 : 1;
   __shared__ float red[WAVES][NACC * MT][256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -222,6 +238,62 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
 #pragma unroll
       for (int j = 0; j < 4; ++j) red[wave][a * MT + mt][lane * 4 + j] = acc[a][mt][j];
   __syncthreads();
+  if (EPI == EPI_ROPE_KV) {
+    // thread e <-> (token m, pair p): the sums of local rows p and p + 8
+    const int tiles_per_head = rk.hd / 16;
+    const int gh = blockIdx.x / tiles_per_head, jt = blockIdx.x % tiles_per_head;  // head among [q heads | k heads | v heads]
+    const bool is_q = gh < rk.heads, is_v = gh >= rk.heads + rk.kv_heads;
+    const int rot_tiles = is_v ? 0 : rk.rot / 16;
+    const bool rotary = jt < rot_tiles;
+    const int half = rk.rot / 2;
+    for (int e = threadIdx.x; e < M * 8; e += WAVES * 64) {
+      const int m = e >> 3, p = e & 7;
+      const int mt = m >> 4, mr = m & 15;
+      // local row r sits at lane (r / 4) * 16 + token, element r % 4
+      const int i1 = ((p >> 2) * 16 + mr) * 4 + (p & 3), i2 = (((p + 8) >> 2) * 16 + mr) * 4 + (p & 3);
+      float x1 = 0.f, x2 = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) {
+        x1 += red[wv][mt][i1];
+        x2 += red[wv][mt][i2];
+      }
+      int d1, d2;
+      if (rotary) {
+        const int j = jt * 8 + p;
+        const float ang = (float)rk.positions[m] * rk.inv_freq[j];
+        const float c = cosf(ang), sn = sinf(ang);
+        const float a = x1, b = x2;
+        x1 = a * c - b * sn;
+        x2 = b * c + a * sn;
+        d1 = j;
+        d2 = j + half;
+      } else {
+        d1 = rk.rot * (is_v ? 0 : 1) + (jt - rot_tiles) * 16 + p;
+        d2 = d1 + 8;
+      }
+      if (is_q) {
+        bf16_t* o = (bf16_t*)out + (size_t)m * out_stride + gh * rk.hd;
+        o[d1] = (bf16_t)x1;
+        o[d2] = (bf16_t)x2;
+      } else if (rk.write_kv) {
+        const int pos = rk.positions[m];
+        const int page = rk.block_table[(size_t)rk.token_req[m] * rk.table_stride + pos / rk.page_size];
+        const int off = pos % rk.page_size;
+        if (!is_v) {
+          const int kh = gh - rk.heads;
+          bf16_t* kd = rk.k_cache + (((size_t)page * rk.page_size + off) * rk.kv_heads + kh) * rk.hd;
+          kd[d1] = (bf16_t)x1;
+          kd[d2] = (bf16_t)x2;
+        } else {
+          const int vh = gh - rk.heads - rk.kv_heads;
+          bf16_t* vd = rk.v_cache + (((size_t)page * rk.kv_heads + vh) * rk.hd) * rk.page_size + off;
+          vd[(size_t)d1 * rk.page_size] = (bf16_t)x1;
+          vd[(size_t)d2 * rk.page_size] = (bf16_t)x2;
+        }
+      }
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < MT * 256; e += WAVES * 64) {
     const int mt = e >> 8, le = e & 255;
     const int l = le >> 2, j = le & 3;
@@ -242,33 +314,36 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
 
 template <int MT, int WAVES>
 static int launch_tiled(void* out, const void* x, const void* w, const void* w2, int M, int N, int K, int x_stride,
-                        int out_stride, int epi, int out_f32, hipStream_t stream) {
+                        int out_stride, int epi, int out_f32, const RopeKvParams& rk, hipStream_t stream) {
   const int grid = (N + 15) / 16;
   const bf16_t* xb = (const bf16_t*)x;
   const bf16_t* wb = (const bf16_t*)w;
   const bf16_t* w2b = (const bf16_t*)w2;
   if (epi == EPI_SILU_MUL) {
     if (out_f32) return NS_ERR_UNSUPPORTED;
-    gemm_tiled_kernel<MT, WAVES, EPI_SILU_MUL, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, w2b, M, N, K, x_stride, out_stride);
+    gemm_tiled_kernel<MT, WAVES, EPI_SILU_MUL, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, w2b, M, N, K, x_stride, out_stride, rk);
+  } else if (epi == EPI_ROPE_KV) {
+    if (out_f32 || MT != 1) return NS_ERR_UNSUPPORTED;
+    gemm_tiled_kernel<1, WAVES, EPI_ROPE_KV, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk);
   } else if (out_f32) {
-    gemm_tiled_kernel<MT, WAVES, EPI_STORE, float><<<grid, WAVES * 64, 0, stream>>>((float*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride);
+    gemm_tiled_kernel<MT, WAVES, EPI_STORE, float><<<grid, WAVES * 64, 0, stream>>>((float*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk);
   } else {
-    gemm_tiled_kernel<MT, WAVES, EPI_STORE, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride);
+    gemm_tiled_kernel<MT, WAVES, EPI_STORE, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk);
   }
   return ns_launch_status();
 }
 
-// wt (and wt2) in the tiled layout described above; N and K are the sizes of the plain matrix.
-extern "C" int ns_gemm_tiled_bf16(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
-                                  int x_stride, int out_stride, int epi, int out_f32, int waves, hipStream_t stream) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
+static int tiled_dispatch(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K, int x_stride,
+                          int out_stride, int epi, int out_f32, int waves, const RopeKvParams& rk, hipStream_t stream) {
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K) return NS_ERR_BAD_ARG;
+  if (epi != EPI_ROPE_KV && out_stride < N) return NS_ERR_BAD_ARG;
   if (epi == EPI_SILU_MUL && !wt2) return NS_ERR_BAD_ARG;
   const int mt = (M + 15) / 16;
 #define NS_TILED(MTV)                                                                                               \
   case MTV:                                                                                                         \
-    return waves == 8 ? launch_tiled<MTV, 8>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, stream)  \
-         : waves == 2 ? launch_tiled<MTV, 2>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, stream)  \
-                      : launch_tiled<MTV, 4>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, stream);
+    return waves == 8 ? launch_tiled<MTV, 8>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, rk, stream)  \
+         : waves == 2 ? launch_tiled<MTV, 2>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, rk, stream)  \
+                      : launch_tiled<MTV, 4>(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, rk, stream);
   switch (mt) {
     NS_TILED(1)
     NS_TILED(2)
@@ -315,4 +390,28 @@ extern "C" int ns_gemm_skinny_bf16(void* out, const void* x, const void* w, cons
   }
 #undef NS_SKINNY
   return NS_ERR_BAD_ARG;
+}
+
+// wt (and wt2) in the tiled layout described above; N and K are the sizes of the plain matrix.
+extern "C" int ns_gemm_tiled_bf16(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
+                                  int x_stride, int out_stride, int epi, int out_f32, int waves, hipStream_t stream) {
+  if (epi != EPI_STORE && epi != EPI_SILU_MUL) return NS_ERR_BAD_ARG;
+  RopeKvParams rk = {};
+  return tiled_dispatch(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, waves, rk, stream);
+}
+
+// The stacked q/k/v product of up to 16 tokens with rotation and cache write fused in.  ``wt`` holds the stacked matrix with
+// its rows permuted as RopeKvParams describes; ``q_out`` [M, >= heads * hd] receives the rotated q.
+extern "C" int ns_gemm_qkv_rope_bf16(void* q_out, const void* x, const void* wt, int M, int K, int x_stride, int q_stride,
+                                     const int* positions, const int* token_req, const int* block_table, int table_stride,
+                                     const float* inv_freq, void* k_cache, void* v_cache, int heads, int kv_heads, int hd,
+                                     int rot, int page_size, int write_kv, int waves, hipStream_t stream) {
+  if (M > 16 || hd % 16 || rot % 16 || rot > hd || heads <= 0 || kv_heads <= 0 || page_size <= 0 || q_stride < heads * hd)
+    return NS_ERR_BAD_ARG;
+  RopeKvParams rk;
+  rk.positions = positions; rk.token_req = token_req; rk.block_table = block_table; rk.inv_freq = inv_freq;
+  rk.k_cache = (bf16_t*)k_cache; rk.v_cache = (bf16_t*)v_cache; rk.table_stride = table_stride; rk.heads = heads;
+  rk.kv_heads = kv_heads; rk.hd = hd; rk.rot = rot; rk.page_size = page_size; rk.write_kv = write_kv;
+  const int N = (heads + 2 * kv_heads) * hd;
+  return tiled_dispatch(q_out, x, wt, nullptr, M, N, K, x_stride, q_stride, EPI_ROPE_KV, 0, waves, rk, stream);
 }

@@ -214,9 +214,13 @@ class TiledWeight:
     wt[rt][kt][i][lane = 16 g + r][e] = w[16 rt + r][128 kt + 32 g + 8 i + e], rows padded to a multiple of 16 and
     k to a multiple of 128 with zeros, so that every load of a wave is one contiguous kilobyte."""
 
-    def __init__(self, w: torch.Tensor) -> None:
+    def __init__(self, w: torch.Tensor, row_order: torch.Tensor | None = None) -> None:
+        """``row_order``: the rows of ``w`` in the order in which they are laid out (a permutation), for kernels whose
+        epilogue wants particular rows together in a tile."""
         if w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_cuda:
             raise KernelRefused("TiledWeight takes a bfloat16 matrix on the GPU")
+        if row_order is not None:
+            w = w[row_order.to(w.device)]
         self.n, self.k = w.shape
         n_pad, k_pad = -(-self.n // 16) * 16, -(-self.k // 128) * 128
         if (n_pad, k_pad) != (self.n, self.k):
@@ -264,6 +268,54 @@ def linear_tiled(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None,
                                            c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(waves), _stream()),
            "linear_tiled")
     return out
+
+
+def qkv_rope_row_order(heads: int, kv_heads: int, head_dim: int, rotary_dim: int) -> torch.Tensor:
+    """The row order of a stacked [q; k; v] matrix for ``linear_qkv_rope``: per head 16-row tiles; in the rotary part of a
+    q or k head a tile holds 8 channels j and their partners j + rotary_dim/2, elsewhere 16 consecutive channels."""
+    order = []
+    half = rotary_dim // 2
+    for g in range(heads + 2 * kv_heads):
+        base = g * head_dim
+        rot = rotary_dim if g < heads + kv_heads else 0
+        for jt in range(rot // 16):
+            order += [base + jt * 8 + e for e in range(8)] + [base + half + jt * 8 + e for e in range(8)]
+        for d0 in range(rot, head_dim, 16):
+            order += [base + d0 + e for e in range(16)]
+    return torch.tensor(order, dtype=torch.int64)
+
+
+def qkv_rope_takes(x: torch.Tensor, head_dim: int, rotary_dim: int) -> bool:
+    return x.dtype == torch.bfloat16 and x.shape[0] <= 16 and head_dim % 16 == 0 and rotary_dim % 16 == 0
+
+
+def linear_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, positions, token_req, block_table, inv_freq, k_cache,
+                    v_cache, heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True, waves: int = 0) -> None:
+    """The stacked q/k/v product of at most 16 tokens with rotation and cache write fused into its epilogue: q goes rotated
+    into ``q_out`` [M, >= heads * head_dim], k rotated into its K page slot, v into the transposed V page.  ``w`` is the
+    stacked matrix tiled in ``qkv_rope_row_order``."""
+    _gpu(x, q_out, positions, token_req, block_table, inv_freq, k_cache, v_cache)
+    m = x.shape[0]
+    if not (tiled_takes(x, w.k) and qkv_rope_takes(x, head_dim, rotary_dim)) or x.shape[1] != w.k:
+        raise KernelRefused("linear_qkv_rope takes at most 16 bfloat16 rows and head and rotary sizes that are multiples of 16")
+    if w.n != (heads + 2 * kv_heads) * head_dim:
+        raise KernelRefused("linear_qkv_rope: the weight does not hold heads + 2 kv_heads heads")
+    if q_out.dtype != torch.bfloat16 or q_out.shape[0] != m or q_out.shape[1] < heads * head_dim or q_out.stride(1) != 1:
+        raise KernelRefused("linear_qkv_rope: q_out must be bfloat16 [rows, >= heads * head_dim]")
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
+    page = k_cache.shape[1]
+    if (k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+            or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("linear_qkv_rope: cache pages do not fit heads, head size or dtype")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2) or positions.numel() != m or token_req.numel() != m:
+        raise KernelRefused("linear_qkv_rope: positions, token_req are per row; inv_freq holds rotary_dim / 2 float32 values")
+    if waves == 0:
+        waves = 8 if w.k >= 2048 else 4
+    _check(build.core().ns_gemm_qkv_rope_bf16(_ptr(q_out), _ptr(x), _ptr(w.data), c_int(m), c_int(w.k), c_int(x.stride(0)),
+                                              c_int(q_out.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
+                                              c_int(block_table.stride(0)), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(heads),
+                                              c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(page),
+                                              c_int(1 if write_kv else 0), c_int(waves), _stream()), "linear_qkv_rope")
 
 
 # ------------------------------------------------------------------------------------------------ attention

@@ -57,9 +57,15 @@ class Attention:
             t = get(name)
             wqkv[at : at + t.shape[0]].copy_(t)
             at += t.shape[0]
-        self.wqkv = LinearWeight(wqkv)
-        self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous())
         self.position.load(get, dtype, device)
+        # for few rows the stacked matrix is streamed by a kernel that rotates and writes the cache in its epilogue; it
+        # wants the rows tiled in an order of its own
+        rot = self.position.rotary_dim
+        self.wqkv_rope = None
+        if dtype == torch.bfloat16 and s.hidden % 8 == 0 and s.head_dim % 16 == 0 and rot % 16 == 0:
+            self.wqkv_rope = ops.TiledWeight(wqkv, ops.qkv_rope_row_order(s.heads, s.kv_heads, s.head_dim, rot))
+        self.wqkv = LinearWeight(wqkv, tiled=self.wqkv_rope is None)
+        self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous())
 
     def cache_need(self):
         return PagedNeed(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
@@ -70,10 +76,15 @@ class Attention:
         pos = self.position
         if pos.max_positions is not None and ctx.max_position >= pos.max_positions:
             raise ValueError(f"position {ctx.max_position} is beyond the model's {pos.max_positions} positions")
-        qkv = self.wqkv(x, out=ctx.arena.take((n, self.wqkv.n), x.dtype))
+        qkv = ctx.arena.take((n, self.wqkv.n), x.dtype)
         table = ctx.block_tables[cache.group]
-        ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
-                          s.head_dim, pos.rotary_dim, write_kv=owns_cache)
+        if self.wqkv_rope is not None and n <= 16 and ops.tiled_takes(x, s.hidden):
+            ops.linear_qkv_rope(x, self.wqkv_rope, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v,
+                                s.heads, s.kv_heads, s.head_dim, pos.rotary_dim, write_kv=owns_cache)
+        else:
+            self.wqkv(x, out=qkv)
+            ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
+                              s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         att = ctx.arena.take((n, s.heads * s.head_dim), x.dtype)
         page = cache.k.shape[1]
         if ops.mfma_attention_takes(x.dtype, s.head_dim, page):

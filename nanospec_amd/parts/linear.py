@@ -21,22 +21,26 @@ STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the sha
 
 
 class LinearWeight:
-    def __init__(self, w: torch.Tensor, keep_plain: bool = True) -> None:
-        """``w``: [out, in] on the GPU in the compute dtype."""
+    def __init__(self, w: torch.Tensor, keep_plain: bool = True, tiled: bool = True) -> None:
+        """``w``: [out, in] on the GPU in the compute dtype.  ``tiled=False``: the caller streams this matrix with a
+        kernel and a layout of its own for few rows, so only the plain layout is kept here."""
         self.n, self.k = w.shape
         self.dtype = w.dtype
-        self.plain = w if (keep_plain or w.dtype != torch.bfloat16 or self.k % 8) else None
-        self.tiled = ops.TiledWeight(w) if (w.dtype == torch.bfloat16 and self.k % 8 == 0) else None
+        fast = w.dtype == torch.bfloat16 and self.k % 8 == 0
+        self.tiled = ops.TiledWeight(w) if (fast and tiled) else None
+        self.plain = w if (keep_plain or self.tiled is None) else None
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False) -> torch.Tensor:
         if x.dtype != self.dtype:
             raise ops.KernelRefused(f"linear: input is {x.dtype}, the weight {self.dtype}")
-        if self.dtype == torch.float32 or self.tiled is None or not ops.tiled_takes(x[:1], self.k):
+        if self.dtype == torch.float32 or self.k % 8 or not ops.tiled_takes(x[:1], self.k):
             return ops.linear_generic(x, self.plain, out=out, out_f32=out_f32)
         m = x.shape[0]
-        if m <= STREAM_ROWS or (m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None)):
+        if self.tiled is not None and (m <= STREAM_ROWS or (m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None))):
             return ops.linear_tiled(x, self.tiled, out=out, out_f32=out_f32)
-        if not out_f32 and self.plain is not None:
+        if self.plain is not None and (not out_f32 or self.tiled is None):
+            if out_f32:
+                return ops.linear_generic(x, self.plain, out=out, out_f32=True)
             return torch.matmul(x, self.plain.t()) if out is None else torch.matmul(x, self.plain.t(), out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)

@@ -195,6 +195,41 @@ def test_rope_kv_write(dtype, rot):
         assert torch.equal(v[pg, :, :, off].cpu(), v0[t])
 
 
+@pytest.mark.parametrize("heads,kvh,hd,rot,page", [(6, 3, 32, 32, 4), (4, 1, 48, 16, 8), (8, 2, 128, 128, 16), (2, 2, 16, 0, 4)])
+def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, page):
+    """One kernel for x @ [Wq; Wk; Wv]^T, the rotation of q and k and the write of k and v into their pages, against the
+    plain product followed by the plain rotation."""
+    ops = _ops()
+    torch.manual_seed(hd + rot)
+    hidden = 72
+    starts, lens = [3, 0, 9], [5, 1, 2]
+    n = sum(lens)
+    table = scattered_tables([s + l for s, l in zip(starts, lens)], page, 16, seed=2).to(DEV)
+    positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    w = (torch.randn((heads + 2 * kvh) * hd, hidden) * 0.3).to(torch.bfloat16)
+    x = torch.randn(n, hidden).to(torch.bfloat16)
+    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot))
+    q_out = torch.zeros(n, (heads + 2 * kvh) * hd, dtype=torch.bfloat16, device=DEV)
+    k, v = make_cache(16, page, kvh, hd, torch.bfloat16)
+    inv = pl.inverse_frequencies(rot, 10000.0, None) if rot else torch.zeros(1)
+    ops.linear_qkv_rope(x.to(DEV), wt, q_out, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot)
+    full = x.float() @ w.float().T  # 32-bit sums: the kernel rotates before it rounds
+    q0 = full[:, : heads * hd].view(n, heads, hd)
+    k0 = full[:, heads * hd : (heads + kvh) * hd].view(n, kvh, hd)
+    v0 = full[:, (heads + kvh) * hd :].view(n, kvh, hd)
+    if rot:
+        cos, sin = pl.rotation_tables(positions.cpu(), inv)
+        q0 = torch.cat([pl.rotate(q0[..., :rot], cos, sin), q0[..., rot:]], -1)
+        k0 = torch.cat([pl.rotate(k0[..., :rot], cos, sin), k0[..., rot:]], -1)
+    assert ulps_of_row_max(q_out[:, : heads * hd].cpu(), q0.reshape(n, -1)).max() <= 1.0
+    for t in range(n):
+        b, p = int(token_req[t]), int(positions[t])
+        pg, off = int(table[b, p // page]), p % page
+        assert ulps_of_row_max(k[pg, off].cpu().reshape(1, -1), k0[t].reshape(1, -1)).max() <= 1.0
+        assert ulps_of_row_max(v[pg, :, :, off].cpu().reshape(1, -1), v0[t].reshape(1, -1)).max() <= 1.0
+
+
 def fill_cache(k, v, table, lens, page, kvh, hd, dtype, seed=0, scale=1.0):
     """Random keys and values for positions [0, len) of every request, written through the block table.
     -> per request (K [len, kvh, hd], V [len, kvh, hd]) on the CPU."""
