@@ -188,8 +188,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
   auto load = [&](Stage& st, int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      st.wf[0][i] = load8(wbase + (size_t)kt * 2048 + i * 512);
-      if (EPI == EPI_SILU_MUL) st.wf[NACC - 1][i] = load8(w2base + (size_t)kt * 2048 + i * 512);
+      st.wf[0][i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wbase + (size_t)kt * 2048 + i * 512));
+      if (EPI == EPI_SILU_MUL) st.wf[NACC - 1][i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w2base + (size_t)kt * 2048 + i * 512));
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) st.xf[mt][i] = load8(xrow[mt] + kt * 128 + i * 8);
     }
