@@ -1,7 +1,8 @@
 """The memory behind the cache manager: pages of keys and values per group of layers, and state slots.
 
 A run-order entry of the model with a ``PagedNeed`` gets one layer of its group's page tensors:
-    K [entries, pages, page, kv_heads, head_dim]       (reference layout, kv/cache.py:16-19)
+    K [entries, pages, kv_heads, page, head_dim]       (the reference keeps [pages, page, kv_heads, head_dim],
+                                                        kv/cache.py:16-19; here a head's part of a page is contiguous)
     V [entries, pages, kv_heads, head_dim, page]       (transposed per page for the attention kernels)
 Both start as zeros: slots that are masked out are still read (reference: kv/cache.py:18).  A page id
 means the same page in every entry of its group.  An entry with a ``StateNeed`` gets a tensor
@@ -51,7 +52,7 @@ class CacheStorage:
         self.group_specs, needs, of_entry = plan_groups(model.cache_needs)
         self.page_size = page_size
         counts = [sum(1 for g in of_entry if g == i) for i in range(len(needs))]
-        self.k = [torch.zeros((counts[i], num_pages[i], page_size, n.kv_heads, n.head_dim), dtype=dtype, device=device)
+        self.k = [torch.zeros((counts[i], num_pages[i], n.kv_heads, page_size, n.head_dim), dtype=dtype, device=device)
                   for i, n in enumerate(needs)]
         self.v = [torch.zeros((counts[i], num_pages[i], n.kv_heads, n.head_dim, page_size), dtype=dtype, device=device)
                   for i, n in enumerate(needs)]
@@ -78,4 +79,4 @@ class CacheStorage:
             t[slot].zero_()
 
     def bytes_per_token(self) -> int:
-        return sum(k[:, 0, 0].numel() * 2 * k.element_size() for k in self.k)
+        return sum(k[:, 0, :, 0].numel() * 2 * k.element_size() for k in self.k)

@@ -6,7 +6,7 @@
 // Query row i of request b stands at position p = kv_len[b] - q_len[b] + i and sees the keys
 // max(0, p - window + 1) .. p  (window == 0: 0 .. p).          (reference: model/attention.py:22-43)
 // Query head h reads key/value head h / (heads / kv_heads).    (reference: model/attention.py:33)
-// K pages: [page][token][kv head][hd];  V pages: [page][kv head][hd][token].
+// K pages: [page][kv head][token][hd];  V pages: [page][kv head][hd][token].
 #include "common.h"
 
 #define AG_THREADS 256
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     float s = -INFINITY;
     if (valid) {
       const int page = table[key / page_size];
-      const T* kr = k_cache + (((size_t)page * page_size + key % page_size) * kv_heads + kvh) * hd;
+      const T* kr = k_cache + (((size_t)page * kv_heads + kvh) * page_size + key % page_size) * hd;
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_f(kr[d]), dot);
       s = dot;

@@ -158,8 +158,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     for (int dt = 0; dt < DT; ++dt) o[u][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int qlo = wlo & ~3, qhi = (whi - 1) & ~3;  // first and last 4-key group that holds a seen key
-  const size_t kv_row = (size_t)a.kv_heads * HD;   // elements per token of a K page
-  const bf16_t* kbase = a.k_cache + (size_t)kvh * HD + (WIDE ? g * 8 : g * 4);
+  const size_t kv_row = (size_t)a.kv_heads * HD;   // elements per token of a page
+  const bf16_t* kbase = a.k_cache + (((size_t)kvh * HD) << psh) + (WIDE ? g * 8 : g * 4);  // K pages: [page][kv head][token][HD]
   const bf16_t* vbase = a.v_cache + (((size_t)kvh * HD + c) << psh);
   constexpr size_t v_step = (size_t)16 * PS;  // elements between channel tiles of a V page
 
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     for (int t = 0; t < 2; ++t) {
       const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);
       const int page = table[key >> psh];
-      const bf16_t* krow = kbase + (((size_t)page << psh) + (key & pmask)) * kv_row;
+      const bf16_t* krow = kbase + (((size_t)page * kv_row) << psh) + (size_t)(key & pmask) * HD;
       if (WIDE) {
 #pragma unroll
         for (int i = 0; i < NQ; ++i) blk.kw[t * NQ + i] = *reinterpret_cast<const bf16x8*>(krow + i * 32);

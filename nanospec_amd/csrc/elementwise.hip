@@ -153,7 +153,9 @@ extern "C" int ns_rmsnorm(void* out, void* resid, const void* x, const void* w, 
 //   qkv row layout: [heads*hd | kv_heads*hd | kv_heads*hd]
 //   pair (j, j + rot/2), j < rot/2:  x_j' = x_j cos - x_{j+rot/2} sin ;  x_{j+rot/2}' = x_{j+rot/2} cos + x_j sin
 //   angle = position * inv_freq[j], all in 32-bit            (reference: model/llama.py:133-136,150-158)
-//   K page layout: [page][token in page][kv head][hd]        (reference: kv/cache.py:16-26)
+//   K page layout: [page][kv head][token in page][hd]        (the reference keeps [page][token][kv head][hd],
+//                                                             kv/cache.py:16-26; here a head's keys of a page are
+//                                                             contiguous, which is how the attention kernels read them)
 //   V page layout: [page][kv head][hd][token in page]        (transposed: the attention kernels read 4 or 8
 //                                                             consecutive tokens of one channel in one load)
 //   page = block_table[req * table_stride + position / page_size]
@@ -189,7 +191,7 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* _
   const int off = pos % page_size;
   const T* krow = row + heads * hd;
   const T* vrow = krow + kv_heads * hd;
-  T* kdst = k_cache + ((size_t)page * page_size + off) * kv_heads * hd;
+  T* kdst = k_cache + (size_t)page * kv_heads * page_size * hd + (size_t)off * hd;
   T* vdst = v_cache + (size_t)page * kv_heads * hd * page_size + off;
   for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x) {
     const int h = e / hd, d = e - h * hd;
@@ -202,7 +204,7 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* _
     } else {
       kv = to_f(krow[e]);
     }
-    kdst[e] = from_f<T>(kv);
+    kdst[(size_t)h * page_size * hd + d] = from_f<T>(kv);
     vdst[(size_t)e * page_size] = vrow[e];
   }
 }

@@ -31,7 +31,7 @@ struct RopeKvParams {
   const int* token_req;    // [M]
   const int* block_table;  // [requests, table_stride]
   const float* inv_freq;   // [rot / 2]
-  bf16_t* k_cache;         // [pages, page, kv_heads, hd]
+  bf16_t* k_cache;         // [pages, kv_heads, page, hd]
   bf16_t* v_cache;         // [pages, kv_heads, hd, page]
   int table_stride, heads, kv_heads, hd, rot, page_size, write_kv;
 };
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
         const int off = pos % rk.page_size;
         if (!is_v) {
           const int kh = gh - rk.heads;
-          bf16_t* kd = rk.k_cache + (((size_t)page * rk.page_size + off) * rk.kv_heads + kh) * rk.hd;
+          bf16_t* kd = rk.k_cache + (((size_t)page * rk.kv_heads + kh) * rk.page_size + off) * rk.hd;
           kd[d1] = (bf16_t)x1;
           kd[d2] = (bf16_t)x2;
         } else {

@@ -104,7 +104,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, token_req: torch.T
                   head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
     """Rotate q in place inside ``qkv`` [N, (heads + 2 kv_heads) * head_dim]; rotate k and write k and v of
     every token into the pages ``block_table[token_req[t], position // page]``.
-    k_cache [pages, page, kv_heads, head_dim]; v_cache [pages, kv_heads, head_dim, page]."""
+    k_cache [pages, kv_heads, page, head_dim]; v_cache [pages, kv_heads, head_dim, page]."""
     _gpu(qkv, positions, token_req, block_table, inv_freq, k_cache, v_cache)
     n = positions.numel()
     width = (heads + 2 * kv_heads) * head_dim
@@ -115,8 +115,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, token_req: torch.T
         raise KernelRefused("rope_kv_write: token_req is per token, block_table is [requests, pages]")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2):
         raise KernelRefused("rope_kv_write: inv_freq must hold rotary_dim/2 float32 values")
-    page = k_cache.shape[1]
-    if (k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+    page = k_cache.shape[2]
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
             or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
         raise KernelRefused("rope_kv_write: cache pages do not fit heads, head size or dtype")
     _check(build.core().ns_rope_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
@@ -303,8 +303,8 @@ def linear_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, positi
     if q_out.dtype != torch.bfloat16 or q_out.shape[0] != m or q_out.shape[1] < heads * head_dim or q_out.stride(1) != 1:
         raise KernelRefused("linear_qkv_rope: q_out must be bfloat16 [rows, >= heads * head_dim]")
     _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
-    page = k_cache.shape[1]
-    if (k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+    page = k_cache.shape[2]
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
             or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
         raise KernelRefused("linear_qkv_rope: cache pages do not fit heads, head size or dtype")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2) or positions.numel() != m or token_req.numel() != m:
@@ -323,8 +323,8 @@ def linear_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, positi
 
 def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim):
     _gpu(q, out, k_cache, v_cache)
-    page = k_cache.shape[1]
-    if (k_cache.dim() != 4 or k_cache.shape[2:] != (kv_heads, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+    page = k_cache.shape[2] if k_cache.dim() == 4 else 0
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
             or not k_cache.is_contiguous() or not v_cache.is_contiguous() or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype):
         raise KernelRefused("attention: cache pages do not fit heads, head size or dtype")
     if q.stride(1) != 1 or q.shape[1] < heads * head_dim:

@@ -86,7 +86,7 @@ class Attention:
             ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
                               s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         att = ctx.arena.take((n, s.heads * s.head_dim), x.dtype)
-        page = cache.k.shape[1]
+        page = cache.k.shape[2]
         if ops.mfma_attention_takes(x.dtype, s.head_dim, page):
             group = s.heads // s.kv_heads
             for plan in ctx.attention_plans(group, s.kv_heads, s.head_dim):

@@ -142,7 +142,7 @@ def test_silu_mul(dtype):
 
 
 def make_cache(pages, page, kvh, hd, dtype):
-    k = torch.zeros(pages, page, kvh, hd, dtype=dtype, device=DEV)
+    k = torch.zeros(pages, kvh, page, hd, dtype=dtype, device=DEV)
     v = torch.zeros(pages, kvh, hd, page, dtype=dtype, device=DEV)
     return k, v
 
@@ -191,7 +191,7 @@ def test_rope_kv_write(dtype, rot):
     for t in range(n):
         b, p = int(token_req[t]), int(positions[t])
         pg, off = int(table[b, p // page]), p % page
-        torch.testing.assert_close(k[pg, off].cpu().float(), k_ref[t].float(), **tol)
+        torch.testing.assert_close(k[pg, :, off].cpu().float(), k_ref[t].float(), **tol)
         assert torch.equal(v[pg, :, :, off].cpu(), v0[t])
 
 
@@ -226,7 +226,7 @@ def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, pa
     for t in range(n):
         b, p = int(token_req[t]), int(positions[t])
         pg, off = int(table[b, p // page]), p % page
-        assert ulps_of_row_max(k[pg, off].cpu().reshape(1, -1), k0[t].reshape(1, -1)).max() <= 1.0
+        assert ulps_of_row_max(k[pg, :, off].cpu().reshape(1, -1), k0[t].reshape(1, -1)).max() <= 1.0
         assert ulps_of_row_max(v[pg, :, :, off].cpu().reshape(1, -1), v0[t].reshape(1, -1)).max() <= 1.0
 
 
@@ -242,7 +242,7 @@ def fill_cache(k, v, table, lens, page, kvh, hd, dtype, seed=0, scale=1.0):
             pg, off = int(table[b, p // page]), p % page
             if pg < 0:
                 continue
-            k[pg, off] = kk[p].to(DEV)
+            k[pg, :, off] = kk[p].to(DEV)
             v[pg, :, :, off] = vv[p].to(DEV)
         out.append((kk, vv))
     return out
@@ -358,7 +358,7 @@ def test_attention_far_key_and_page_edges(kernel):
         q = torch.randn(1, heads * hd, dtype=dtype, device=DEV)
         pg, off = int(table[0, special // page]), special % page
         for h in range(kvh):
-            k[pg, off, h] = (q.view(heads, hd)[h * (heads // kvh)] * 4).to(dtype)  # aligned with the group's first query head
+            k[pg, h, off] = (q.view(heads, hd)[h * (heads // kvh)] * 4).to(dtype)  # aligned with the group's first query head
         starts, lens = [total - 1], [1]
         if kernel == "mfma":
             out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd)

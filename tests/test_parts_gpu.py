@@ -108,7 +108,7 @@ def test_attention_part_with_cache_across_steps(dtype, window):
     part.load(ws.__getitem__, dtype, DEV)
     need = part.cache_need()
     assert (need.kv_heads, need.head_dim, need.window) == (kvh, hd, window)
-    k = torch.zeros(12, page, kvh, hd, dtype=dtype, device=DEV)
+    k = torch.zeros(12, kvh, page, hd, dtype=dtype, device=DEV)
     v = torch.zeros(12, kvh, hd, page, dtype=dtype, device=DEV)
     cache = PagedView(0, k, v)
     xs = [torch.randn(21, hidden).to(dtype), torch.randn(14, hidden).to(dtype)]
