@@ -1,0 +1,194 @@
+// bfloat16 matrix products on the matrix cores for 17 to 64 rows (decode at large batch, short portions):
+//   out[M, N] = x[M, K] . w[N, K]^T,  32-bit accumulation, weights in the tiled layout of gemm_bf16.hip.
+//
+// With this many rows the traffic of x counts: a workgroup of 4 waves owns 64 rows of w (16 per wave) and all its
+// waves walk through the same k tiles, so that a tile of x (64 tokens x 128 k) is fetched once per workgroup, with
+// whole-row loads, into LDS and read from there by every wave in the layout the matrix instruction wants.  The weights
+// still go from memory straight into registers, each exactly once.  Since 64 rows per workgroup leave too few workgroups
+// to fill the GPU, K is cut into `ksplit` ranges over blockIdx.y; each range writes 32-bit partial sums and a second
+// kernel adds the ranges in order and applies the epilogue (store as bfloat16 or 32-bit, or silu(gate) * up).
+// (reference for the products: the nn.Linear calls of model/llama.py:175,184,195,286)
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+#define WIDE_XPAD 8                  // elements of padding per row of the x tile in LDS
+#define WIDE_XROW (128 + WIDE_XPAD)  // elements per row
+
+// partial[(a * ksplit + s) * M * N + m * N + n]: sum over k range s of matrix a (0: w, 1: w2)
+// NT: 16-row tiles of w per wave (64 NT rows per workgroup); each fragment of x read from LDS serves all of them.
+template <int MT, int NACC, int NT>
+__global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ partial, const bf16_t* __restrict__ x,
+                                                        const bf16_t* __restrict__ wt, const bf16_t* __restrict__ wt2,
+                                                        int M, int N, int K, int x_stride, int ksplit) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][WIDE_XROW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int KT = (K + 127) / 128;
+  const int row_tiles = (N + 15) / 16;
+  const int rt = (blockIdx.x * 4 + wave) * NT;  // first of this wave's row tiles
+  const bool has_rows = rt < row_tiles;
+  const int split = blockIdx.y;
+  const int per = (KT + ksplit - 1) / ksplit;
+  const int kt0 = split * per, kt1 = min(KT, kt0 + per);
+
+  const bf16_t* wbase = wt + (size_t)(has_rows ? rt : 0) * KT * 2048 + lane * 8;
+  const bf16_t* w2base = NACC == 2 ? wt2 + (size_t)(has_rows ? rt : 0) * KT * 2048 + lane * 8 : nullptr;
+
+  const size_t tile_step = (size_t)KT * 2048;  // elements between consecutive row tiles
+  bool tile_ok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) tile_ok[t] = rt + t < row_tiles;
+  f32x4 acc[NACC][NT][MT];
+#pragma unroll
+  for (int a = 0; a < NACC; ++a)
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[a][t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // The x tile of one k tile: MT*16 rows of 128 k = MT*16*16 pieces of 8; 256 threads take MT pieces each: thread t
+  // takes piece t % 16 of rows t / 16 + 16 j, so 16 consecutive threads read one row's 256 contiguous bytes.
+  const int xrow0 = tid >> 4, xcol = (tid & 15) * 8;
+  // A stage holds what one k tile needs from memory: this wave's fragments of w (and w2) and this thread's pieces of x.
+  // DEPTH stages are in flight: the loads of k tile t + DEPTH - 1 are issued before the arithmetic of k tile t.
+  constexpr int DEPTH = NACC * NT >= 2 ? 2 : 3;
+  struct Stage {
+    bf16x8 wf[NACC][NT][4];
+    bf16x8 xr[MT];
+  };
+  Stage st[DEPTH];
+  auto fetch = [&](Stage& sg, int kt) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const size_t off = (tile_ok[t] ? t * tile_step : 0) + (size_t)kt * 2048;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sg.wf[0][t][i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wbase + off + i * 512));
+        if (NACC == 2) sg.wf[1][t][i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w2base + off + i * 512));
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const int m = xrow0 + 16 * j;
+      const int k = kt * 128 + xcol;
+      sg.xr[j] = (m < M && k < K) ? *reinterpret_cast<const bf16x8*>(x + (size_t)m * x_stride + k) : zero;
+    }
+  };
+  auto step = [&](const Stage& sg, int buf) {
+    // x pieces into LDS, then every wave multiplies its w fragments with the whole tile.  One barrier per k tile: a
+    // wave that writes buffer b for tile t + 2 has passed the barrier of tile t + 1, which every wave reaches only
+    // after it has finished reading b for tile t.
+#pragma unroll
+    for (int j = 0; j < MT; ++j) *reinterpret_cast<bf16x8*>(&xs[buf][xrow0 + 16 * j][xcol]) = sg.xr[j];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][mt * 16 + r][g * 32 + i * 8]);
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[a][t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sg.wf[a][t][i], xf, acc[a][t][mt], 0, 0, 0);
+      }
+  };
+
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (kt0 + d < kt1) fetch(st[d], kt0 + d);
+  for (int kt = kt0; kt < kt1; kt += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int cur = kt + d;
+      if (cur < kt1) {
+        if (cur + DEPTH - 1 < kt1) fetch(st[(d + DEPTH - 1) % DEPTH], cur + DEPTH - 1);
+        step(st[d], (cur - kt0) & 1);
+      }
+    }
+  }
+
+  if (!has_rows) return;
+  // acc[a][t][mt][j] is the sum for w row 16 (rt + t) + 4 g + j and token 16 mt + r
+#pragma unroll
+  for (int a = 0; a < NACC; ++a)
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + r, n = (rt + t) * 16 + g * 4;
+        if (m >= M || !tile_ok[t]) continue;
+        float* dst = partial + ((size_t)(a * ksplit + split) * M + m) * N + n;
+        if (n + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<f32x4*>(dst) = acc[a][t][mt];
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (n + j < N) dst[j] = acc[a][t][mt][j];
+        }
+      }
+}
+
+// out[m][n] = epilogue(sum_s partial[s][m][n]); ranges are added in order.
+template <typename OutT, int SILU>
+__global__ void gemm_wide_reduce_kernel(OutT* __restrict__ out, const float* __restrict__ partial, int M, int N, int out_stride,
+                                        int ksplit) {
+  const size_t total = (size_t)M * N;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    float s = 0.f, u = 0.f;
+    for (int k = 0; k < ksplit; ++k) {
+      s += partial[(size_t)k * total + e];
+      if (SILU) u += partial[(size_t)(ksplit + k) * total + e];
+    }
+    if (SILU) s = s / (1.f + expf(-s)) * u;
+    const size_t m = e / N;
+    out[m * out_stride + (e - m * N)] = (OutT)s;
+  }
+}
+
+template <int MT>
+static int launch_wide(float* partial, const bf16_t* x, const bf16_t* wt, const bf16_t* wt2, int M, int N, int K, int x_stride,
+                       int ksplit, int nt, hipStream_t stream) {
+  const int row_tiles = (N + 15) / 16;
+  dim3 grid((row_tiles + 4 * nt - 1) / (4 * nt), ksplit);
+  if (wt2 && nt == 2)
+    gemm_wide_kernel<MT, 2, 2><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit);
+  else if (wt2)
+    gemm_wide_kernel<MT, 2, 1><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit);
+  else if (nt == 2)
+    gemm_wide_kernel<MT, 1, 2><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit);
+  else
+    gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit);
+  return ns_launch_status();
+}
+
+// workspace: (wt2 ? 2 : 1) * ksplit * M * N floats.  epi 0: store; 1: silu(x.w^T) * (x.w2^T).
+extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
+                                 int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, hipStream_t stream) {
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N || !workspace) return NS_ERR_BAD_ARG;
+  if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
+  const int KT = (K + 127) / 128;
+  if (ksplit < 1 || ksplit > KT || ksplit > 65535 || (nt != 1 && nt != 2)) return NS_ERR_BAD_ARG;
+  const int mt = (M + 15) / 16;
+  float* part = (float*)workspace;
+  int st;
+  switch (mt) {
+    case 1: st = launch_wide<1>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
+    case 2: st = launch_wide<2>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
+    case 3: st = launch_wide<3>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
+    default: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
+  }
+  if (st != NS_OK) return st;
+  const size_t total = (size_t)M * N;
+  const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+  if (epi == 1)
+    gemm_wide_reduce_kernel<bf16_t, 1><<<blocks, 256, 0, stream>>>((bf16_t*)out, part, M, N, out_stride, ksplit);
+  else if (out_f32)
+    gemm_wide_reduce_kernel<float, 0><<<blocks, 256, 0, stream>>>((float*)out, part, M, N, out_stride, ksplit);
+  else
+    gemm_wide_reduce_kernel<bf16_t, 0><<<blocks, 256, 0, stream>>>((bf16_t*)out, part, M, N, out_stride, ksplit);
+  return ns_launch_status();
+}

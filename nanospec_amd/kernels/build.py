@@ -27,7 +27,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
-CORE_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attn_generic.hip", "sampling.hip", "gemm_bf16.hip", "graph.hip"]
+CORE_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attn_generic.hip", "sampling.hip", "gemm_bf16.hip", "gemm_wide.hip", "graph.hip"]
 ATTN_SOURCES = ["attn_mfma.hip"]
 
 _loaded: dict[str, ctypes.CDLL] = {}

@@ -270,6 +270,46 @@ def linear_tiled(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None,
     return out
 
 
+def wide_plan(n: int, k: int) -> tuple[int, int]:
+    """(ranges K is cut into, 16-row tiles per wave) of ``linear_wide``: two tiles per wave when there are rows enough,
+    then enough ranges that the workgroups fill the GPU, with at least four k tiles of 128 per range."""
+    nt = 2 if n >= 8192 else 1
+    row_groups = -(-n // (64 * nt))
+    k_tiles = -(-k // 128)
+    return max(1, min(16, k_tiles // 4, round(640 / row_groups))), nt
+
+
+def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
+                out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0) -> torch.Tensor:
+    """bfloat16 x @ w.T for up to 64 rows from a tiled weight, with the tile of x shared through LDS by the four waves of
+    a workgroup and K cut into ``ksplit`` ranges that a second kernel adds up; with ``w2``: silu(x @ w.T) * (x @ w2.T).
+    ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values."""
+    _gpu(x, out, workspace)
+    if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k):
+        raise KernelRefused(f"linear_wide takes bfloat16 x [rows <= {SKINNY_MAX_ROWS}, {w.k}] with an inner size that is a "
+                            f"multiple of 8; got {tuple(x.shape)} {x.dtype}")
+    m = x.shape[0]
+    want = torch.float32 if out_f32 else x.dtype
+    if out is None:
+        out = torch.empty((m, w.n), dtype=want, device=x.device)
+    if out.shape != (m, w.n) or out.dtype != want or out.stride(1) != 1:
+        raise KernelRefused("linear_wide: out has the wrong shape or dtype")
+    if w2 is not None and (w2.n != w.n or w2.k != w.k or out_f32):
+        raise KernelRefused("linear_wide: w2 must match w and the gated result is bfloat16")
+    plan = wide_plan(w.n, w.k)
+    ksplit, nt = ksplit or plan[0], nt or plan[1]
+    need = (2 if w2 is not None else 1) * ksplit * m * w.n
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+    if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+        raise KernelRefused("linear_wide: workspace too small")
+    _check(build.core().ns_gemm_wide_bf16(_ptr(out), _ptr(workspace), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None),
+                                          c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
+                                          c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), _stream()),
+           "linear_wide")
+    return out
+
+
 def qkv_rope_row_order(heads: int, kv_heads: int, head_dim: int, rotary_dim: int) -> torch.Tensor:
     """The row order of a stacked [q; k; v] matrix for ``linear_qkv_rope``: per head 16-row tiles; in the rotary part of a
     q or k head a tile holds 8 channels j and their partners j + rotary_dim/2, elsewhere 16 consecutive channels."""

@@ -82,7 +82,7 @@ class Attention:
             ops.linear_qkv_rope(x, self.wqkv_rope, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v,
                                 s.heads, s.kv_heads, s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         else:
-            self.wqkv(x, out=qkv)
+            self.wqkv(x, out=qkv, arena=ctx.arena)
             ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
                               s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         att = ctx.arena.take((n, s.heads * s.head_dim), x.dtype)
@@ -96,7 +96,7 @@ class Attention:
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)
-        return self.wo(att, out=out)
+        return self.wo(att, out=out, arena=ctx.arena)
 
 
 registry.register("mixer", "attention", Attention)

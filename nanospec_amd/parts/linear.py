@@ -5,9 +5,10 @@ matrix-core mode of reduced precision is ever used).
 
 bfloat16: decode and short portions (up to ``STREAM_ROWS`` rows) run the hand-written matrix-core kernel that streams
 the weights once; it reads them in a layout re-laid at load time (``kernels.ops.TiledWeight``) in which every load
-of a wave is one contiguous kilobyte.  More rows go to the platform's GEMM library on the plain layout, as the
-reference's nn.Linear does (model/llama.py:168-171).  32-bit results (logits) always come from the streaming kernel,
-in slices of 64 rows, so that no logit is rounded to bfloat16.  Both layouts are kept in memory unless
+of a wave is one contiguous kilobyte.  17 to 64 rows run a second hand-written kernel on the same layout (x shared
+through LDS, K cut into ranges) where it is ahead of the library.  More rows go to the platform's GEMM library on the
+plain layout, as the reference's nn.Linear does (model/llama.py:168-171).  32-bit results (logits) always come from the
+hand-written kernels, in slices of 64 rows, so that no logit is rounded to bfloat16.  Both layouts are kept in memory unless
 ``keep_plain=False``.
 """
 
@@ -18,6 +19,8 @@ import torch
 from ..kernels import ops
 
 STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured (see profiles/)
+WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
+#                    32-bit results, which the library does not give); wider products go to the library
 
 
 class LinearWeight:
@@ -30,23 +33,33 @@ class LinearWeight:
         self.tiled = ops.TiledWeight(w) if (fast and tiled) else None
         self.plain = w if (keep_plain or self.tiled is None) else None
 
-    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False, arena=None) -> torch.Tensor:
+        """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated."""
         if x.dtype != self.dtype:
             raise ops.KernelRefused(f"linear: input is {x.dtype}, the weight {self.dtype}")
         if self.dtype == torch.float32 or self.k % 8 or not ops.tiled_takes(x[:1], self.k):
             return ops.linear_generic(x, self.plain, out=out, out_f32=out_f32)
         m = x.shape[0]
-        if self.tiled is not None and (m <= STREAM_ROWS or (m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None))):
+        if self.tiled is not None and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled, out=out, out_f32=out_f32)
+        if self.tiled is not None and m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None or self.n <= WIDE_MAX_N):
+            ksplit, nt = ops.wide_plan(self.n, self.k)
+            ws = arena.take((ksplit * m * self.n,), torch.float32) if arena is not None else None
+            return ops.linear_wide(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
         if self.plain is not None and (not out_f32 or self.tiled is None):
             if out_f32:
                 return ops.linear_generic(x, self.plain, out=out, out_f32=True)
             return torch.matmul(x, self.plain.t()) if out is None else torch.matmul(x, self.plain.t(), out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
+        ksplit, nt = ops.wide_plan(self.n, self.k)
+        ws = arena.take((ksplit * ops.SKINNY_MAX_ROWS * self.n,), torch.float32) if arena is not None else None
         for s in range(0, m, ops.SKINNY_MAX_ROWS):
             e = min(m, s + ops.SKINNY_MAX_ROWS)
-            ops.linear_tiled(x[s:e], self.tiled, out=out[s:e], out_f32=out_f32)
+            if e - s <= STREAM_ROWS:
+                ops.linear_tiled(x[s:e], self.tiled, out=out[s:e], out_f32=out_f32)
+            else:
+                ops.linear_wide(x[s:e], self.tiled, out=out[s:e], out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
         return out
 
 
@@ -62,12 +75,16 @@ class GatedWeights:
 
     def __call__(self, ctx, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         m = x.shape[0]
-        if self.tiled is not None and ops.tiled_takes(x[:1], self.k) and (m <= STREAM_ROWS or (self.stacked is None and m <= ops.SKINNY_MAX_ROWS)):
+        fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
+        if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
-        if self.stacked is None:
+        if fast and self.stacked is None:
+            # (with the plain layout at hand the library's product plus the activation kernel is faster from 17 rows on)
+            ksplit, nt = ops.wide_plan(self.inter, self.k)
+            ws = ctx.arena.take((2 * ksplit * min(m, ops.SKINNY_MAX_ROWS) * self.inter,), torch.float32)
             for s in range(0, m, ops.SKINNY_MAX_ROWS):
                 e = min(m, s + ops.SKINNY_MAX_ROWS)
-                ops.linear_tiled(x[s:e], self.tiled[0], w2=self.tiled[1], out=out[s:e])
+                ops.linear_wide(x[s:e], self.tiled[0], w2=self.tiled[1], out=out[s:e], workspace=ws, ksplit=ksplit, nt=nt)
             return out
         gu = ctx.arena.take((m, 2 * self.inter), x.dtype)
         if self.dtype == torch.float32 or self.k % 8:

@@ -85,4 +85,4 @@ class DecoderModel:
         (reference: model/llama.py:284-286, engine/engine.py:382)."""
         n = rows.numel()
         h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
-        return self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True)
+        return self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True, arena=ctx.arena)

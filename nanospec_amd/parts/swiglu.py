@@ -33,7 +33,7 @@ class SwiGLU:
 
     def forward(self, ctx, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         act = self.gate_up(ctx, x, out=ctx.arena.take((x.shape[0], self.spec.intermediate), x.dtype))
-        return self.down(act, out=out)
+        return self.down(act, out=out, arena=ctx.arena)
 
 
 registry.register("ffn", "swiglu", SwiGLU)

@@ -118,6 +118,31 @@ def test_linear_tiled(m, n, k):
         torch.testing.assert_close(part.cpu(), ref[:, 16:48], rtol=1e-4, atol=1e-3 * math.sqrt(k))
 
 
+@pytest.mark.parametrize("m", [17, 33, 48, 64, 5])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064), (4096, 14336)])
+def test_linear_wide(m, n, k):
+    """The kernel for 17 to 64 rows: x through LDS, K cut into ranges; every count of ranges, sizes off the tile."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m + 3, k + 8, dtype=torch.bfloat16, device=DEV)[:m, :k]  # a strided view of a wider buffer
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    wt, wt2 = ops.TiledWeight(w), ops.TiledWeight(w2)
+    ref = x.cpu().float() @ w.cpu().float().T
+    k_tiles = -(-k // 128)
+    for ks in sorted({1, 2, min(5, k_tiles), k_tiles, 0} - {k_tiles + 1}):
+        if ks > k_tiles:
+            continue
+        for nt in (1, 2):
+            out = ops.linear_wide(x, wt, out_f32=True, ksplit=ks, nt=nt)
+            torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
+    assert ulps_of_row_max(ops.linear_wide(x, wt).cpu(), ref).max() <= 1.0
+    u = x.cpu().float() @ w2.cpu().float().T
+    for nt in (1, 2):
+        act = ops.linear_wide(x, wt, w2=wt2, nt=nt)
+        assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0
+
+
 def test_linear_skinny_refuses():
     ops = _ops()
     from nanospec_amd.kernels import KernelRefused

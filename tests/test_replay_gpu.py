@@ -156,3 +156,50 @@ def test_trace_run_program(tiny_folders, tmp_path):
                 continue
             got = torch.from_file(str(path), size=len(w) * vocab, dtype=torch.float32).view(len(w), vocab)
             check(got, torch.stack([ref[rid][p] for rid, p in w]), dtype, f"trace_run step {step['step']}")
+
+
+# ------------------------------------------------------------------------------------------------ a real shape
+
+
+@pytest.fixture(scope="module")
+def llama_1b_slice(tmp_path_factory):
+    """Two layers of the Llama-3.2-1B shape (width 2048, 32 heads over 8 key/value heads of 64, feed-forward 8192,
+    vocabulary 128256, tied head, llama3 scaling with factor 32), random weights."""
+    from nanospec_amd.config import LlamaConfig
+    from nanospec_amd.weights import write_model_folder
+
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0,
+               max_position_embeddings=131072, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    return write_model_folder(tmp_path_factory.mktemp("llama1b") / "m", LlamaConfig.from_hf(cfg), seed=3, dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_real_shape_slice_matches_plain(llama_1b_slice, dtype):
+    """The kernels at the sizes of a real model (head size 64, a vocabulary of 128256, width 2048): one request whole with
+    its last tokens decoded, one in portions, mixed in one batch, at positions where the llama3 scaling matters."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.loader import load_model
+
+    folder = llama_1b_slice
+    cfg, w = pl.read_config(folder), pl.read_weights(folder, dtype)
+    seqs = {"a": random_tokens(150, 128256, 1), "b": random_tokens(83, 128256, 2)}
+    ref = {r: pl.logits_of_sequence(w, cfg, t, dtype) for r, t in seqs.items()}
+    model = load_model(folder, dtype=dtype)
+    rep = Replayer(model, 384, page_size=16)
+
+    def step(entries, end=()):
+        out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(wants)} for r, s, e, wants in entries], list(end))
+        want = torch.cat([ref[r][s:e][list(wants)] for r, s, e, wants in entries])
+        check(out, want, dtype, str([(r, s, e) for r, s, e, _ in entries]))
+
+    step([("a", 0, 130, [0, 64, 129])])
+    step([("a", 130, 131, [0]), ("b", 0, 37, [36])])
+    step([("a", 131, 132, [0]), ("b", 37, 39, [0, 1])])
+    for p in range(132, 150):
+        q = 39 + (p - 132) * 2
+        step([("a", p, p + 1, [0]), ("b", q, q + 2, [0, 1])], end=["a"] if p == 149 else [])
+    step([("b", 75, 83, list(range(8)))], end=["b"])
+    rep.manager.check()
