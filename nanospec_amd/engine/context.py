@@ -8,6 +8,8 @@ kv_indptr / kv_indices / kv_last_page_len / positions / slots):
     qo_indptr[B+1] kv_lens[B] state_slots[B]      per request; kv_lens counts the keys after this step
     want_rows[R]                                  token rows whose logits are wanted
     patch_dst[P] patch_src[P]                     token rows whose ids come from a device tensor of the step before
+    sample_opts[4, S]                             temperature, top_p, uniform number (float bits) and top_k of the rows that a
+                                                  captured step samples itself
     chunk tiles [Tc, 8]                           requests with more than one token, 32 tokens per tile; a tile is
     decode tiles [Td, 8]                          (request, first token, first row, tokens, keys, 0, 0, 0); decode
                                                   tiles are the requests with exactly one token
@@ -34,14 +36,14 @@ class BatchLayout:
     """Offsets of the fields inside the int32 buffer for given sizes."""
 
     def __init__(self, n_tokens: int, n_reqs: int, n_want: int, n_chunk_tiles: int, n_decode_tiles: int, n_groups: int,
-                 table_width: int, n_patch: int = 0) -> None:
+                 table_width: int, n_patch: int = 0, n_sample: int = 0) -> None:
         self.N, self.B, self.R, self.Tc, self.Td, self.G, self.P = n_tokens, n_reqs, n_want, n_chunk_tiles, n_decode_tiles, n_groups, table_width
         off = 0
         self.fields = {}
         for name, size in (("token_ids", n_tokens), ("positions", n_tokens), ("token_req", n_tokens), ("qo_indptr", n_reqs + 1),
                            ("kv_lens", n_reqs), ("state_slots", n_reqs), ("want_rows", n_want),
                            ("ctiles", TILE_INTS * n_chunk_tiles), ("dtiles", TILE_INTS * n_decode_tiles),
-                           ("patch_dst", n_patch), ("patch_src", n_patch)):
+                           ("patch_dst", n_patch), ("patch_src", n_patch), ("sample_opts", 4 * n_sample)):
             self.fields[name] = (off, size)
             off += _pad4(max(size, 1))
         self.table_off = []

@@ -134,20 +134,29 @@ class Engine:
         else:
             row_of = {id(w.req): i for i, w in enumerate(token_src["sampling"])}
             entries = [StepEntry(w.req.id, [0], [0]) for w in work]
-            device_tokens = (token_src["sampled"][0][0], [(j, row_of[id(w.req)]) for j, w in enumerate(work)])
+            device_tokens = (token_src["sampled"][0][0], [(j, row_of[id(w.req)]) for j, w in enumerate(work)])  # row 0: the tokens
         samples = [w.samples for w in work] if token_src is None else [True] * len(work)
-        logits = self.runner.step(entries, device_tokens)
+        sampling = [w for w, smp in zip(work, samples) if smp]
+        # one uniform per request and step from its own generator (reference: engine/engine.py:283)
+        uniforms = [float(torch.rand(1, generator=w.req.gen)) for w in sampling]
+        in_graph = ([w.req.params for w in sampling], uniforms) if len(sampling) == len(work) else None
+        logits = self.runner.step(entries, device_tokens, sampling=in_graph)
         self._mark("forward")
         for w in work:
             w.req.computed += w.n
-        sampling = [w for w, smp in zip(work, samples) if smp]
         sampled, staged, kept = [], [], []
-        if sampling:
+        if sampling and self.runner.last_sampled is not None:  # the captured step sampled as well
+            buf, n = self.runner.last_sampled
+            with torch.cuda.stream(self.runner.stream):
+                sampled.append(buf)
+                staged.append(self._stage.stage(buf, n))
+                if self.config.record_logits:
+                    kept.append(logits.cpu())
+        elif sampling:
             with torch.cuda.stream(self.runner.stream):
                 for s in range(0, len(sampling), self.config.head_chunk):
                     chunk = sampling[s : s + self.config.head_chunk]
-                    # one uniform per request and step from its own generator (reference: engine/engine.py:283)
-                    u = [float(torch.rand(1, generator=w.req.gen)) for w in chunk]
+                    u = uniforms[s : s + len(chunk)]
                     rows = logits[s : s + len(chunk)]
                     sampled.append(launch_sample(rows, [w.req.params for w in chunk], u, self._stage))
                     staged.append(self._stage.stage(sampled[-1]))

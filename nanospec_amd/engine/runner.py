@@ -41,14 +41,22 @@ class _DecodeGraph:
     def __init__(self, runner: "ModelRunner", size: int) -> None:
         self.size = size
         n_groups = len(runner.manager.groups)
-        self.layout = BatchLayout(size, size, size, 0, size, n_groups, runner.table_width, n_patch=size)
+        self.layout = BatchLayout(size, size, size, 0, size, n_groups, runner.table_width, n_patch=size, n_sample=size)
         dev = runner.device
         self.dev_buf = torch.zeros(self.layout.total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
         self.host_np = self.host.numpy()
         self.arena = Arena(dev)  # grows during the warm-up run, then stays as it is
         self.logits: torch.Tensor | None = None
+        self.sampled = torch.zeros((3, size), dtype=torch.int32, device=dev)  # what the captured sampling kernel writes
         self.graph = None
+
+    def sample_options(self):
+        """Views of the batch buffer: (temperature, top_p, uniform) float32 and top_k int32, one per row."""
+        off, n = self.layout.fields["sample_opts"]
+        opts = self.dev_buf[off : off + n].view(4, self.size)
+        f = opts[:3].view(torch.float32)
+        return f[0], f[1], f[2], opts[3]
 
     def context(self, runner) -> StepContext:
         return StepContext(self.layout, self.dev_buf, self.arena, max_position=0, max_kv_len=runner.table_width * runner.page_size,
@@ -77,6 +85,7 @@ class ModelRunner:
         self._pad_ready = False
         self._staged: torch.cuda.Event | None = None
         self.last_used_graph = False
+        self.last_sampled = None
 
     # ------------------------------------------------------------------ requests
 
@@ -108,13 +117,18 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ the step
 
-    def step(self, entries: list[StepEntry], device_tokens=None) -> torch.Tensor | None:
+    def step(self, entries: list[StepEntry], device_tokens=None, sampling=None) -> torch.Tensor | None:
         """Run one batch.  -> float32 logits [number of wanted places, vocab] in the order of the entries
         and of their ``want`` lists, or None if nothing is wanted.  Nothing here waits for the GPU.
 
         ``device_tokens`` = (int32 tensor on the GPU, [(entry index, row of the tensor), ...]): the first token id of
         those entries is taken from the tensor when the step runs (the id in ``tokens`` is a placeholder), so that a
-        step can be enqueued before the step that samples its input has finished."""
+        step can be enqueued before the step that samples its input has finished.
+
+        ``sampling`` = ([SamplingParams per entry], [uniform number per entry]): if the step replays a captured graph the
+        graph samples too, and ``last_sampled`` is then (int32 [3, bucket] on the GPU, rows that count); otherwise
+        ``last_sampled`` is None and the caller samples from the returned logits."""
+        self.last_sampled = None
         if not entries:
             return None
         vocab = self.model.spec.vocab_size
@@ -144,7 +158,7 @@ class ModelRunner:
             self._staged.synchronize()  # the last batch has left the pinned staging buffers
         with torch.cuda.stream(self.stream):
             if self.use_graphs and all(n == 1 for n in lens) and n_want and self._bucket(len(entries)) is not None:
-                logits = self._step_graph(entries, rcs, starts, device_tokens)
+                logits = self._step_graph(entries, rcs, starts, device_tokens, sampling)
                 self.last_used_graph = True
             else:
                 logits = self._step_eager(entries, rcs, starts, lens, n_want, device_tokens)
@@ -227,7 +241,7 @@ class ModelRunner:
             self._mirror(self.manager.get(PAD_REQUEST))
             self._pad_ready = True
 
-    def _fill_graph(self, g: _DecodeGraph, entries, rcs, starts, device_tokens=None) -> None:
+    def _fill_graph(self, g: _DecodeGraph, entries, rcs, starts, device_tokens=None, sampling=None) -> None:
         """Real rows first, then pad rows that read and write the reserved pad page at position 0
         (reference: engine/graphs.py:115-167)."""
         pad = self.manager.get(PAD_REQUEST)
@@ -239,6 +253,19 @@ class ModelRunner:
         fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables)
         if device_tokens:
             self._put_patch(g.host_np, g.layout, [e for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
+        off, n = g.layout.fields["sample_opts"]
+        opts = g.host_np[off : off + n].reshape(4, g.size)
+        opts[:] = 0  # pad rows: temperature 0
+        if sampling is not None:
+            params, uniforms = sampling
+            k = len(params)
+            f = opts[:3].view(np.float32)
+            f[0, :k] = [p.temperature for p in params]
+            f[1, :k] = [p.top_p for p in params]
+            f[2, :k] = uniforms
+            opts[3, :k] = [p.top_k for p in params]
+        else:
+            opts[:3].view(np.float32)[1] = 1.0
         g.dev_buf.copy_(g.host, non_blocking=True)
         self._staged = torch.cuda.Event()
         self._staged.record(self.stream)
@@ -253,7 +280,10 @@ class ModelRunner:
         def run():
             g.arena.reset()
             resid, delta = self.model.forward_hidden(ctx, self.storage.views)
-            return self.model.logits(ctx, resid, delta, ctx.want_rows)
+            logits = self.model.logits(ctx, resid, delta, ctx.want_rows)
+            temp, top_p, uni, top_k = g.sample_options()
+            ops.sample(logits, temp, uni, top_k=top_k, top_p=top_p, out=g.sampled)
+            return logits
 
         run()  # warm-up: loads the libraries and lets the arena grow to what a step needs
         self.stream.synchronize()
@@ -266,7 +296,7 @@ class ModelRunner:
         self._graphs[size] = g
         return g
 
-    def _step_graph(self, entries, rcs, starts, device_tokens=None):
+    def _step_graph(self, entries, rcs, starts, device_tokens=None, sampling=None):
         self._ensure_pad()
         size = self._bucket(len(entries))
         g = self._graphs.get(size) or self._capture(size)
@@ -274,8 +304,10 @@ class ModelRunner:
         if -(-max_kv // self.page_size) > self.table_width:
             raise ValueError("a request is longer than the block tables of the captured graphs")
         self._check_positions(max_kv - 1)
-        self._fill_graph(g, entries, rcs, starts, device_tokens)
+        self._fill_graph(g, entries, rcs, starts, device_tokens, sampling)
         g.graph.launch()
+        if sampling is not None and all(e.want for e in entries):
+            self.last_sampled = (g.sampled, len(entries))
         rows = [i for i, e in enumerate(entries) if e.want]
         if len(rows) == len(entries):
             return g.logits[: len(entries)]

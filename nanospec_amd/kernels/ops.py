@@ -438,11 +438,11 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, top_k: torch.Tensor | None = None,
-           top_p: torch.Tensor | None = None):
-    """Per row of float32 ``logits``: arg-max when temperature is 0, else a draw by inverse CDF with the
-    row's uniform number.  -> (token int32, log-probability of it under the raw logits, log-probability
-    under the processed distribution; 0 for arg-max rows)."""
-    _gpu(logits, temperature, uniform, top_k, top_p)
+           top_p: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Per row of float32 ``logits``: arg-max when temperature is 0, else a draw by inverse CDF with the row's uniform
+    number.  -> int32 [3, rows]: row 0 the tokens, row 1 the bits of the float32 log-probability of the token under the
+    raw logits, row 2 the bits of its float32 log-probability under the processed distribution (0 for arg-max rows)."""
+    _gpu(logits, temperature, uniform, top_k, top_p, out)
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelRefused("sample: logits must be float32 [rows, vocab]")
     rows, vocab = logits.shape
@@ -450,12 +450,18 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
                         ("top_k", top_k, torch.int32), ("top_p", top_p, torch.float32)):
         if t is not None and (t.dtype != dt or t.numel() != rows or not t.is_contiguous()):
             raise KernelRefused(f"sample: {name} must hold one {dt} per row")
-    tok = torch.empty(rows, dtype=torch.int32, device=logits.device)
-    lp = torch.empty(rows, dtype=torch.float32, device=logits.device)
-    slp = torch.empty(rows, dtype=torch.float32, device=logits.device)
-    _check(build.core().ns_sample(_ptr(tok), _ptr(lp), _ptr(slp), _ptr(logits), c_int(logits.stride(0)), _ptr(temperature),
+    if out is None:
+        out = torch.empty((3, rows), dtype=torch.int32, device=logits.device)
+    if out.dtype != torch.int32 or out.shape != (3, rows) or not out.is_contiguous():
+        raise KernelRefused("sample: out must be a contiguous int32 [3, rows]")
+    _check(build.core().ns_sample(_ptr(out[0]), _ptr(out[1]), _ptr(out[2]), _ptr(logits), c_int(logits.stride(0)), _ptr(temperature),
                                   _ptr(top_k), _ptr(top_p), _ptr(uniform), c_int(rows), c_int(vocab), _stream()), "sample")
-    return tok, lp, slp
+    return out
+
+
+def unpack_sample(packed: torch.Tensor):
+    """int32 [3, rows] of ``sample`` -> (tokens int32, log-probabilities float32, processed log-probabilities float32)."""
+    return packed[0], packed[1].view(torch.float32), packed[2].view(torch.float32)
 
 
 # ------------------------------------------------------------------------------------------------ graphs

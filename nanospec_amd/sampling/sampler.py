@@ -14,8 +14,8 @@ from .params import SamplingParams, TokenInfo
 
 
 def launch_sample(logits: torch.Tensor, params: list[SamplingParams], uniforms: list[float], stage: "SampleStage | None" = None):
-    """logits float32 [rows, vocab] on the GPU -> (token int32, raw log-probability, processed log-probability) tensors
-    on the GPU.  Waits for nothing: with a ``stage`` the options travel through pinned memory (a copy from ordinary host
+    """logits float32 [rows, vocab] on the GPU -> int32 [3, rows] on the GPU (tokens, bits of the raw log-probability,
+    bits of the processed log-probability; see ``kernels.ops.sample``).  Waits for nothing: with a ``stage`` the options travel through pinned memory (a copy from ordinary host
     memory would wait for everything enqueued before it)."""
     dev = logits.device
     rows = logits.shape[0]
@@ -63,29 +63,31 @@ class SampleStage:
         if base.numel() == 4 * self.rows:
             self._options.append((base, ev))
 
-    def stage(self, sampled):
-        tok, lp, slp = sampled
-        n = tok.numel()
-        host = self.free.pop() if self.free else torch.empty(3 * max(self.rows, n), dtype=torch.float32).pin_memory()
-        host[: 3 * n].copy_(torch.stack([tok.to(torch.float32), lp, slp]).view(-1), non_blocking=True)
+    def stage(self, sampled: torch.Tensor, rows: int | None = None):
+        """``sampled``: int32 [3, width] on the GPU, contiguous; the first ``rows`` of each line count."""
+        width = sampled.shape[1]
+        host = self.free.pop() if self.free else torch.empty(3 * max(self.rows, width), dtype=torch.int32).pin_memory()
+        host[: 3 * width].copy_(sampled.view(-1), non_blocking=True)
         done = torch.cuda.Event()
-        done.record(torch.cuda.current_stream(tok.device))
-        return host, n, done
+        done.record(torch.cuda.current_stream(sampled.device))
+        return host, (width, width if rows is None else rows), done
 
     def read(self, staged) -> list[TokenInfo]:
         """The step's one wait for the GPU (reference: the single ``.tolist()`` of engine/engine.py:403)."""
-        host, n, done = staged
+        host, (width, n), done = staged
         done.synchronize()
-        packed = host[: 3 * n].view(3, n).tolist()
+        tok = host[:n].tolist()
+        lp = host[width : 3 * width].view(torch.float32).tolist()
         if host.numel() == 3 * self.rows:
             self.free.append(host)
-        return [TokenInfo(int(packed[0][i]), packed[1][i], packed[2][i]) for i in range(n)]
+        return [TokenInfo(tok[i], lp[i], lp[width + i]) for i in range(n)]
 
 
-def read_sample(sampled) -> list[TokenInfo]:
-    tok, lp, slp = sampled
-    packed = torch.stack([tok.to(torch.float32), lp, slp]).tolist()
-    return [TokenInfo(int(packed[0][i]), packed[1][i], packed[2][i]) for i in range(tok.numel())]
+def read_sample(sampled: torch.Tensor) -> list[TokenInfo]:
+    n = sampled.shape[1]
+    host = sampled.cpu()
+    tok, lp, slp = host[0].tolist(), host[1].view(torch.float32).tolist(), host[2].view(torch.float32).tolist()
+    return [TokenInfo(tok[i], lp[i], slp[i]) for i in range(n)]
 
 
 def sample_rows(logits: torch.Tensor, params: list[SamplingParams], uniforms: list[float]) -> list[TokenInfo]:

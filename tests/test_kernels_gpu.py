@@ -434,7 +434,7 @@ def test_sample_greedy_and_temperature():
     z[2, 100] = z[2, 900] = z[2].max() + 1  # a tie: the lowest index wins
     T = torch.tensor([0.0, 0.8, 0.0, 1.0, 0.7, 1.3], device=DEV)
     u = torch.tensor([0.3, 0.9, 0.5, 0.0, 0.5, 0.9999], device=DEV)
-    tok, lp, slp = ops.sample(z, T, u)
+    tok, lp, slp = ops.unpack_sample(ops.sample(z, T, u))
     zc = z.cpu()
     for r in range(rows):
         t = float(T[r])
@@ -459,7 +459,7 @@ def test_sample_top_k_top_p():
     p = torch.tensor([1.0, 0.8, 0.5, 0.2], device=DEV)
     for uu in (0.01, 0.37, 0.62, 0.999):
         u = torch.full((4,), uu, device=DEV)
-        tok, lp, slp = ops.sample(z, T, u, top_k=k, top_p=p)
+        tok, lp, slp = ops.unpack_sample(ops.sample(z, T, u, top_k=k, top_p=p))
         for r in range(4):
             ref_lp = pl.processed_logprobs(z[r].cpu(), float(T[r]), int(k[r]), float(p[r]))
             ref = pl.draw_token(ref_lp, uu)
