@@ -80,14 +80,17 @@ struct KVBlock {
 
 // QT: tiles of 16 columns per wave (2 only with hp == 1: 32 tokens of one head share every load of K and V).
 // PREFETCH: the loads of the next key block are issued before the arithmetic of the current one.
-template <int QT, bool PREFETCH>
+// COOP: the four waves of a workgroup share one tile and one key range and take its 32-key blocks in turn; their
+// results meet in LDS.  Decode is bound by the latency of a wave's chain of loads, so the chain is made four times
+// shorter without more work for the kernel that joins the ranges.
+template <int QT, bool PREFETCH, bool COOP>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int G = a.heads / a.kv_heads;
   const int hblks = (G + a.hp - 1) / a.hp;
   const int ny = a.kv_heads * hblks;
-  const long item = (long)blockIdx.x * 4 + wave;
+  const long item = COOP ? (long)blockIdx.x : (long)blockIdx.x * 4 + wave;
   if (item >= (long)a.n_tiles * a.splits * ny) return;
   const int y = (int)(item % ny);
   const long ts = item / ny;
@@ -163,13 +166,24 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   const bf16_t* vbase = a.v_cache + (((size_t)kvh * HD + c) << psh);
   constexpr size_t v_step = (size_t)16 * PS;  // elements between channel tiles of a V page
 
+  // The page ids of up to 64 consecutive pages are held one per lane and handed round by lane exchange, so that the
+  // chain of loads of a block is one load long (keys and values) rather than two (block table, then keys and values).
+  const int last_page = max(whi - 1, 0) >> psh;
+  int page_base = 0x40000000, my_page = 0;
+  auto page_of = [&](int key) { return __shfl(my_page, (key >> psh) - page_base, 64); };
+
   // Issue the loads of block kb.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
   auto load = [&](KVBlock& blk, int kb) {
     const int key_base = kb * 32;
+    const int p_lo = key_base >> psh, p_hi = (key_base + 31) >> psh;
+    if (p_lo < page_base || p_hi >= page_base + 64) {  // uniform over the wave
+      page_base = p_lo;
+      my_page = table[min(page_base + lane, last_page)];
+    }
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);
-      const int page = table[key >> psh];
+      const int page = page_of(key);
       const bf16_t* krow = kbase + (((size_t)page * kv_row) << psh) + (size_t)(key & pmask) * HD;
       if (WIDE) {
 #pragma unroll
@@ -183,8 +197,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     // for j >= 4, in both operands.
     const int k0 = min(max(key_base + g * 4, qlo), qhi);
     const int k1 = min(max(key_base + 16 + g * 4, qlo), qhi);
-    const bf16_t* v0 = vbase + (((size_t)table[k0 >> psh] * kv_row) << psh) + (k0 & pmask);
-    const bf16_t* v1 = vbase + (((size_t)table[k1 >> psh] * kv_row) << psh) + (k1 & pmask);
+    const bf16_t* v0 = vbase + (((size_t)page_of(k0) * kv_row) << psh) + (k0 & pmask);
+    const bf16_t* v1 = vbase + (((size_t)page_of(k1) * kv_row) << psh) + (k1 & pmask);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       blk.v[dt][0] = *reinterpret_cast<const bf16x4*>(v0 + dt * v_step);
@@ -266,16 +280,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     }
   };
 
+  constexpr int KSTEP = COOP ? 4 : 1;  // blocks between two blocks of this wave
   if (PREFETCH) {
     KVBlock ba, bb;
-    int kb = kb0;
+    int kb = kb0 + (COOP ? wave : 0);
     if (kb < kb1) load(ba, kb);
-    while (kb + 1 < kb1) {
-      load(bb, kb + 1);
+    while (kb + KSTEP < kb1) {
+      load(bb, kb + KSTEP);
       compute(ba, kb);
-      if (kb + 2 < kb1) load(ba, kb + 2);
-      compute(bb, kb + 1);
-      kb += 2;
+      if (kb + 2 * KSTEP < kb1) load(ba, kb + 2 * KSTEP);
+      compute(bb, kb + KSTEP);
+      kb += 2 * KSTEP;
     }
     if (kb < kb1) compute(ba, kb);
   } else {
@@ -284,6 +299,40 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       load(ba, kb);
       compute(ba, kb);
     }
+  }
+
+  if constexpr (COOP) {
+    // Lane l of every wave holds the same columns and channels, so the waves' results are joined lane by lane:
+    // o = sum_w o_w 2^((m_w - m*) scale), likewise the sums, m* = max_w m_w; waves are added in order by wave 0.
+    __shared__ float co[4][DT][64][4];
+    __shared__ float cml[4][2][64];
+    static_assert(QT == 1, "cooperative waves hold one tile");
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(co[wave][dt][lane]) = o[0][dt];
+    cml[wave][0][lane] = m[0];
+    cml[wave][1][lane] = lsum[0];
+    __syncthreads();
+    if (wave != 0) return;
+    float mstar = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mstar = fmaxf(mstar, cml[w][0][lane]);
+    const float msafe = mstar == -INFINITY ? 0.f : mstar;
+    float l = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float wgt = fast_exp2((cml[w][0][lane] - msafe) * a.scale_log2);
+      l += cml[w][1][lane] * wgt;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(co[w][dt][lane]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[0][dt][j] += v[j] * wgt;
+      }
+    }
+    m[0] = mstar;
+    lsum[0] = l;
   }
 
 #pragma unroll
@@ -377,14 +426,14 @@ extern "C" int ns_attn_mfma_page_size() { return PS; }
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
-                            hipStream_t stream) {
+                            int coop, hipStream_t stream) {
   if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size != PS || window < 0 ||
       splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
     return NS_ERR_BAD_ARG;
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
   if (!(scale > 0.f)) return NS_ERR_BAD_ARG;  // maxima are tracked on unscaled scores
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
-  if (qt != 1 && !(qt == 2 && hp == 1 && splits == 1)) return NS_ERR_BAD_ARG;
+  if (qt != 1 && !(qt == 2 && hp == 1 && splits == 1 && !coop)) return NS_ERR_BAD_ARG;
   AttnParams a;
   a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
   a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
@@ -394,12 +443,14 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   a.scale_log2 = scale * 1.4426950408889634f;
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);
-  const long blocks = (items + 3) / 4;
+  const long blocks = coop ? items : (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
   if (qt == 2)
-    attn_mfma_kernel<2, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
+    attn_mfma_kernel<2, false, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
+  else if (coop)
+    attn_mfma_kernel<1, true, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
   else
-    attn_mfma_kernel<1, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
+    attn_mfma_kernel<1, true, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
   const int st = ns_launch_status();
   if (st != NS_OK || splits == 1) return st;
   if (heads > 65535) return NS_ERR_BAD_ARG;

@@ -60,6 +60,7 @@ class AttentionPlan:
     splits: int
     workspace: tuple | None
     qt: int = 1
+    coop: bool = False
 
 
 class StepContext:
@@ -95,15 +96,17 @@ class StepContext:
             hp = 1
             while hp < min(group, 16):
                 hp *= 2
+            # decode is bound by the latency of each wave's chain of loads: the four waves of a workgroup share a tile, and
+            # the keys are cut into ranges until about a thousand waves are at work
             items = lay.Td * kv_heads * -(-group // hp)
-            splits = max(1, min(32, -(-1024 // items)))
+            splits = max(1, min(16, 1024 // (4 * items)))
             if not self.fixed_splits:
-                splits = max(1, min(splits, -(-self.max_kv_len // 128)))
+                splits = max(1, min(splits, -(-self.max_kv_len // 256)))
             ws = None
             if splits > 1:
                 cols = lay.Td * (16 // hp) * kv_heads * group
                 ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
-            plans.append(AttentionPlan(self._dtiles, hp, splits, ws))
+            plans.append(AttentionPlan(self._dtiles, hp, splits, ws, coop=True))
         return plans
 
 

@@ -400,12 +400,13 @@ TILE_INTS = 8  # ints per attention tile descriptor: request, first token, first
 
 def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_heads: int, head_dim: int, scale: float,
                    window: int = 0, hp: int = 1, splits: int = 1,
-                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1) -> torch.Tensor:
+                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1, coop: bool = False) -> torch.Tensor:
     """bfloat16 attention on the matrix cores for the tiles described in ``tiles`` (int32 [n_tiles, 8]: request, first
     token of the tile among the request's tokens of this step, row of the request's first token in ``q``, tokens of the
     request in this step, keys after this step, three zeros).  ``hp`` heads of a group times 16/hp tokens make a tile;
     with ``qt`` = 2 (only with hp = 1 and no splits) a tile is 32 tokens.  ``splits`` > 1 cuts the keys of every tile
-    into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors."""
+    into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors.  With ``coop`` the four
+    waves of a workgroup share each tile and range (for decode, where a wave's chain of loads is what takes the time)."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
     if not mfma_attention_takes(q.dtype, head_dim, page):
         raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
@@ -416,8 +417,8 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
         raise KernelRefused(f"attention_mfma: tiles must be int32 [n_tiles, {TILE_INTS}], 16-byte aligned")
     if hp not in (1, 2, 4, 8, 16):
         raise KernelRefused("attention_mfma: hp is a power of two up to 16")
-    if qt != 1 and not (qt == 2 and hp == 1 and splits == 1):
-        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1 and no splits")
+    if qt != 1 and not (qt == 2 and hp == 1 and splits == 1 and not coop):
+        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1, no splits and no cooperating waves")
     n_tiles = tiles.shape[0]
     po = pm = None
     if splits > 1:
@@ -430,7 +431,8 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     lib = build.attn(head_dim, page)
     _check(lib.ns_attn_mfma(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tiles),
                             _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads),
-                            c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), _stream()), "attention_mfma")
+                            c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_int(1 if coop else 0), _stream()),
+           "attention_mfma")
     return out
 
 

@@ -92,7 +92,7 @@ class Attention:
             for plan in ctx.attention_plans(group, s.kv_heads, s.head_dim):
                 ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim,
                                    s.softmax_scale, window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace,
-                                   qt=plan.qt)
+                                   qt=plan.qt, coop=plan.coop)
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)

@@ -323,7 +323,7 @@ def test_attention_generic(dtype, case, heads, kvh, hd, page):
         assert ulps_of_row_max(out.cpu(), ref).max() <= 4  # the reference's bound, tests/test_backends.py:71
 
 
-def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2):
+def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False):
     n = sum(lens)
     indptr = [0]
     for l in lens:
@@ -344,7 +344,7 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
         cols = len(dt) * (16 // hp) * heads
         ws = (torch.empty(cols * splits * hd, dtype=torch.float32, device=DEV), torch.empty(cols * splits * 2, dtype=torch.float32, device=DEV))
         ops.attention_mfma(q, out, k, v, i32(dt), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=hp,
-                           splits=splits, workspace=ws if splits > 1 else None)
+                           splits=splits, workspace=ws if splits > 1 else None, coop=coop)
     return out
 
 
@@ -362,10 +362,10 @@ def test_attention_mfma(case, heads, kvh, hd, page):
     n = sum(lens)
     q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
-    for splits, qt in ((1, 2), (3, 1), (7, 2), (33, 1)):
-        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt)
+    for splits, qt, coop in ((1, 2, False), (3, 1, False), (7, 2, True), (33, 1, False), (1, 1, True), (2, 2, True)):
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt, coop=coop)
         u = ulps_of_row_max(out.cpu(), ref).max()
-        assert u <= 4, f"{case} splits={splits} qt={qt}: {u:.2f} ulps"
+        assert u <= 4, f"{case} splits={splits} qt={qt} coop={coop}: {u:.2f} ulps"
 
 
 @pytest.mark.parametrize("kernel", ["generic", "mfma"])
