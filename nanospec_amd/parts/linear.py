@@ -18,7 +18,7 @@ import torch
 
 from ..kernels import ops
 
-STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured (see profiles/)
+STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured
 WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
 #                    32-bit results, which the library does not give); wider products go to the library
 
