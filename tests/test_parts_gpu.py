@@ -1,6 +1,7 @@
 """Each kind of part alone against the plain function it implements, at sizes of its own; a model put together from
 parts in an unusual order (a layer run twice, an entry that reads another entry's cache); and a toy mixer with state of
-its own that is defined here, registered, built and stepped without touching the framework."""
+its own, a toy feed-forward with routing and a toy position encoding that are defined here, registered, built and stepped
+without touching the framework."""
 
 from __future__ import annotations
 
@@ -262,3 +263,136 @@ def test_toy_mixer_with_state_layer_twice_and_borrowed_cache():
     step([("a", 11, 30), ("c", 0, 2)])                  # request c gets the slot request b gave back: it must start from zero
     step([("a", 30, 37), ("c", 2, 29)], end=["a", "c"])
     rep.manager.check()
+
+
+# ------------------------------------------------------- a toy feed-forward with routing and a toy position encoding
+
+
+@dataclass(frozen=True)
+class HarmonicRotationSpec:
+    """Rotation of the first ``rotary_dim`` channels of a head by angle position / (j + 1) for pair j."""
+
+    kind: ClassVar[str] = "harmonic"
+    rotary_dim: int
+
+
+class HarmonicRotation:
+    graph_safe = True
+    max_positions = None
+
+    def __init__(self, spec, prefix=""):
+        self.rotary_dim, self.inv_freq = spec.rotary_dim, None
+
+    def wanted(self):
+        return {}
+
+    def load(self, get, dtype, device):
+        self.inv_freq = (1.0 / torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float32)).to(device)
+
+
+@dataclass(frozen=True)
+class TopOneExpertsSpec:
+    """Each token goes through the one expert (a SwiGLU) its router row likes best, weighted by that expert's share of
+    the soft-max over the router's 32-bit logits."""
+
+    kind: ClassVar[str] = "top_one"
+    hidden: int
+    inner: int
+    experts: int
+
+
+class TopOneExperts:
+    graph_safe = False
+
+    def __init__(self, spec, prefix):
+        self.spec, self.prefix = spec, prefix
+
+    def wanted(self):
+        s, p = self.spec, self.prefix
+        out = {p + "router.weight": ((s.experts, s.hidden), "linear")}
+        for e in range(s.experts):
+            out[f"{p}experts.{e}.gate.weight"] = ((s.inner, s.hidden), "linear")
+            out[f"{p}experts.{e}.up.weight"] = ((s.inner, s.hidden), "linear")
+            out[f"{p}experts.{e}.down.weight"] = ((s.hidden, s.inner), "linear")
+        return out
+
+    def load(self, get, dtype, device):
+        from nanospec_amd.parts.linear import GatedWeights, LinearWeight
+
+        p = self.prefix
+        self.router = get(p + "router.weight").to(device=device, dtype=torch.float32)
+        on = lambda name: get(name).to(device=device, dtype=dtype).contiguous()
+        self.gated = [GatedWeights(on(f"{p}experts.{e}.gate.weight"), on(f"{p}experts.{e}.up.weight")) for e in range(self.spec.experts)]
+        self.down = [LinearWeight(on(f"{p}experts.{e}.down.weight")) for e in range(self.spec.experts)]
+
+    def forward(self, ctx, x, out=None):
+        share = torch.softmax(x.float() @ self.router.T, dim=-1)
+        top, choice = share.max(-1)
+        res = torch.zeros_like(x)
+        for e in range(self.spec.experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                xe = x[rows].contiguous()
+                y = self.down[e](self.gated[e](ctx, xe, torch.empty((rows.numel(), self.spec.inner), dtype=x.dtype, device=x.device)))
+                res[rows] = (y.float() * top[rows, None]).to(x.dtype)
+        return res if out is None else out.copy_(res)
+
+
+def test_toy_routed_feed_forward_and_toy_position_in_one_layer_only():
+    import math
+
+    from nanospec_amd.config.spec import AttentionSpec, LayerCall, ModelSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.parts import DecoderModel, register
+    from nanospec_amd.weights import DictSource, random_tensors
+
+    register("ffn", "top_one", TopOneExperts)
+    register("position", "harmonic", HarmonicRotation)
+    hidden, vocab, hd = 40, 61, 32
+    norm = RMSNormSpec(hidden, 1e-5)
+    layers = (PreNormBlockSpec("model.layers.0.", norm, AttentionSpec(hidden, 2, 2, hd, RopeSpec(hd, 1e4), 1 / math.sqrt(hd)), norm, SwiGLUSpec(hidden, 56)),
+              PreNormBlockSpec("model.layers.1.", norm, AttentionSpec(hidden, 2, 1, hd, HarmonicRotationSpec(16), 0.25), norm, TopOneExpertsSpec(hidden, 24, 3)))
+    spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers, (LayerCall(0), LayerCall(1)), norm, "model.norm.weight", "lm_head.weight", False)
+    net = DecoderModel(spec)
+    wanted = net.wanted()
+    assert "model.layers.1.top_one.router.weight" in wanted and "model.layers.0.mlp.gate_proj.weight" in wanted
+    w = random_tensors(wanted, seed=11)
+    w = {k: v * (8.0 if "proj" in k or "experts" in k or "router" in k else 1.0) for k, v in w.items()}
+    model = net.load(DictSource(w), torch.float32, DEV)
+
+    def plain(tokens):
+        t = len(tokens)
+        x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        positions = torch.arange(t)
+        tables = [pl.rotation_tables(positions, pl.inverse_frequencies(hd, 1e4, None)),
+                  pl.rotation_tables(positions, 1.0 / torch.arange(1, 9, dtype=torch.float32))]
+        for i, (heads, kvh, rot, scale) in enumerate(((2, 2, hd, 1 / math.sqrt(hd)), (2, 1, 16, 0.25))):
+            p = f"model.layers.{i}."
+            h = pl.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+            cos, sin = tables[i]
+            turn = lambda y: torch.cat([pl.rotate(y[..., :rot], cos, sin), y[..., rot:]], -1)
+            q = turn(pl.linear(h, w[p + "self_attn.q_proj.weight"]).view(t, heads, hd))
+            k = turn(pl.linear(h, w[p + "self_attn.k_proj.weight"]).view(t, kvh, hd))
+            v = pl.linear(h, w[p + "self_attn.v_proj.weight"]).view(t, kvh, hd)
+            a = pl.causal_attention(q * (scale * math.sqrt(hd)), k, v).reshape(t, -1)  # the plain function scales by 1/sqrt(d)
+            x = x + pl.linear(a, w[p + "self_attn.o_proj.weight"])
+            h = pl.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+            if i == 0:
+                x = x + pl.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+            else:
+                share = torch.softmax(h @ w[p + "top_one.router.weight"].T, -1)
+                top, choice = share.max(-1)
+                y = torch.stack([pl.swiglu(h[j : j + 1], w[f"{p}top_one.experts.{e}.gate.weight"], w[f"{p}top_one.experts.{e}.up.weight"],
+                                           w[f"{p}top_one.experts.{e}.down.weight"])[0] for j, e in enumerate(choice.tolist())])
+                x = x + y * top[:, None]
+        return pl.rms_norm(x, w["model.norm.weight"], 1e-5) @ w["lm_head.weight"].T
+
+    g = torch.Generator().manual_seed(3)
+    seqs = {r: torch.randint(0, vocab, (n,), generator=g).tolist() for r, n in (("a", 41), ("b", 19))}
+    refs = {r: plain(t) for r, t in seqs.items()}
+    rep = Replayer(model, 128, page_size=8)
+    for entries in ([("a", 0, 17), ("b", 0, 2)], [("a", 17, 18), ("b", 2, 19)], [("a", 18, 41)]):
+        out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(range(e - s))} for r, s, e in entries], [])
+        want = torch.cat([refs[r][s:e] for r, s, e in entries])
+        err = ((out.cpu() - want).abs().amax(-1) / want.abs().amax(-1)).max()
+        assert err < 1e-4, (entries, float(err))
