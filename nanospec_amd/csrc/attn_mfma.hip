@@ -172,14 +172,19 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   int page_base = 0x40000000, my_page = 0;
   auto page_of = [&](int key) { return __shfl(my_page, (key >> psh) - page_base, 64); };
 
-  // Issue the loads of block kb.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
-  auto load = [&](KVBlock& blk, int kb) {
+  // Issue the loads of block kb: keys, values.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked
+  // anyway.
+  auto pages_for = [&](int kb) {
     const int key_base = kb * 32;
     const int p_lo = key_base >> psh, p_hi = (key_base + 31) >> psh;
     if (p_lo < page_base || p_hi >= page_base + 64) {  // uniform over the wave
       page_base = p_lo;
       my_page = table[min(page_base + lane, last_page)];
     }
+  };
+  auto load_k = [&](KVBlock& blk, int kb) {
+    const int key_base = kb * 32;
+    pages_for(kb);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int key = min(max(key_base + t * 16 + c, wlo), whi - 1);
@@ -193,6 +198,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
         for (int i = 0; i < NQ; ++i) blk.kn[t * NQ + i] = *reinterpret_cast<const s16x4*>(krow + i * 16);
       }
     }
+  };
+  auto load_v = [&](KVBlock& blk, int kb) {
+    const int key_base = kb * 32;
+    pages_for(kb);
     // Slot 8 g + j of the second product holds key key_base + 4 g + j for j < 4 and key_base + 16 + 4 g + (j - 4)
     // for j >= 4, in both operands.
     const int k0 = min(max(key_base + g * 4, qlo), qhi);
@@ -205,15 +214,16 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       blk.v[dt][1] = *reinterpret_cast<const bf16x4*>(v1 + dt * v_step);
     }
   };
+  auto load = [&](KVBlock& blk, int kb) {
+    load_k(blk, kb);
+    load_v(blk, kb);
+  };
 
-  auto compute = [&](const KVBlock& blk, int kb) {
-    const int key_base = kb * 32;
-    // every key of the block is seen by every column: no masks needed (uniform over the wave)
-    const bool full = key_base + 31 <= full_hi && key_base >= full_lo;
-    bf16x8 pf[QT];
+  // The three phases of a block: scores S^T = K Q^T; soft-max weights of the block (and the rescaling of what has been
+  // summed so far); O^T += V^T P^T.
+  auto scores = [&](const KVBlock& blk, f32x4 (&s)[QT][2]) {
 #pragma unroll
-    for (int u = 0; u < QT; ++u) {
-      f32x4 s[2];
+    for (int u = 0; u < QT; ++u)
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -224,24 +234,31 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 #pragma unroll
           for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.kn[t * NQ + i], qn[u][i], acc, 0, 0, 0);
         }
-        s[t] = acc;
+        s[u][t] = acc;
       }
-      // s[t][j] is key key_base + 16 t + 4 g + j of column c
+  };
+  auto soften = [&](f32x4 (&s)[QT][2], int kb, bf16x8 (&pf)[QT]) {
+    const int key_base = kb * 32;
+    // every key of the block is seen by every column: no masks needed (uniform over the wave)
+    const bool full = key_base + 31 <= full_hi && key_base >= full_lo;
+#pragma unroll
+    for (int u = 0; u < QT; ++u) {
+      // s[u][t][j] is key key_base + 16 t + 4 g + j of column c
       float mx = -INFINITY;
       // m[u] is the running maximum of the raw scores (the scale is positive); p = 2^((s - m) scale log2 e)
       if (full) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[t][j]);
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][t][j]);
       } else {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int key = key_base + t * 16 + g * 4 + j;
-            const float v = (key >= lo[u] && key <= pos[u]) ? s[t][j] : -INFINITY;
-            s[t][j] = v;
+            const float v = (key >= lo[u] && key <= pos[u]) ? s[u][t][j] : -INFINITY;
+            s[u][t][j] = v;
             mx = fmaxf(mx, v);
           }
       }
@@ -258,7 +275,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = fast_exp2(fmaf(s[t][j], a.scale_log2, shift));
+          const float p = fast_exp2(fmaf(s[u][t][j], a.scale_log2, shift));
           psum += p;
           pf[u][t * 4 + j] = (bf16_t)p;
         }
@@ -271,6 +288,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       }
       lsum[u] += psum;
     }
+  };
+  auto weigh = [&](const KVBlock& blk, const bf16x8 (&pf)[QT]) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       const bf16x4 lo4 = blk.v[dt][0], hi4 = blk.v[dt][1];
@@ -278,6 +297,13 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 #pragma unroll
       for (int u = 0; u < QT; ++u) o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
     }
+  };
+  auto compute = [&](const KVBlock& blk, int kb) {
+    f32x4 s[QT][2];
+    bf16x8 pf[QT];
+    scores(blk, s);
+    soften(s, kb, pf);
+    weigh(blk, pf);
   };
 
   constexpr int KSTEP = COOP ? 4 : 1;  // blocks between two blocks of this wave
@@ -294,10 +320,18 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     }
     if (kb < kb1) compute(ba, kb);
   } else {
+    // One set of registers, two loads in flight: the values of a block are asked for before its scores are formed, and
+    // the keys of the next block as soon as the scores have read this block's keys.
     KVBlock ba;
+    if (kb0 < kb1) load_k(ba, kb0);
     for (int kb = kb0; kb < kb1; ++kb) {
-      load(ba, kb);
-      compute(ba, kb);
+      f32x4 s[QT][2];
+      bf16x8 pf[QT];
+      load_v(ba, kb);
+      scores(ba, s);
+      if (kb + 1 < kb1) load_k(ba, kb + 1);
+      soften(s, kb, pf);
+      weigh(ba, pf);
     }
   }
 
@@ -358,6 +392,274 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       if (g == 0) {
         a.part_ml[(pcol * a.splits + split) * 2] = m[u] * a.scale_log2;  // in the exponent's units
         a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum[u];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Prompt portions when the head size is a multiple of 32 and a page holds 8 tokens or more: a workgroup owns 32 tokens
+// of up to four query heads of one key/value head, one head per wave.  The four waves need the same keys and values,
+// so each block of 32 keys is fetched once per workgroup, a quarter by each wave, and handed round through LDS;
+// the next block is on its way from memory (and its page ids one block further ahead) while this one is used.
+//   keys in LDS:   row 16 t + 4 a + b holds key 8 a + 4 t + b of the block, so that the scores a lane gets from the
+//                  two 16-key products are those of keys 8 g .. 8 g + 7: the order in which it then needs the values
+//   values in LDS: [channel][32 keys], as the pages hold them
+// Rows are padded by 16 bytes, which spreads the 16 rows of one load over all banks.
+// ------------------------------------------------------------------------------------------------
+constexpr bool SHARED_OK = WIDE && PS >= 8;
+constexpr int KROW = HD + 8;               // elements of a key's row in LDS
+constexpr int VROW = 32 + 8;               // elements of a channel's row in LDS
+constexpr int CHUNKS = 32 * HD / 8;        // 16-byte pieces of a block's keys; as many of its values
+constexpr int PER_THREAD = (CHUNKS + 255) / 256;
+constexpr int CPR = PS / 8 < 4 ? PS / 8 : 4;  // 16-byte pieces of a block that lie side by side in a channel's row of a page
+
+// Two waves per SIMD: with more registers the compiler parks the sums in accumulation registers and moves them to and
+// fro around every rescaling.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnParams a) {
+  if constexpr (SHARED_OK) {
+    __shared__ __align__(16) bf16_t lk[2][32 * KROW];
+    __shared__ __align__(16) bf16_t lv[2][HD * VROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int G = a.heads / a.kv_heads;
+    const int hblks = (G + 3) / 4;
+    const int ny = a.kv_heads * hblks;
+    const int y = blockIdx.x % ny;
+    // Tiles are listed in the order of the tokens and the last ones see the most keys.  The first half of the workgroups
+    // takes the later half of the tiles, longest first, the second half the earlier tiles, shortest first: two
+    // workgroups that are half a grid apart, which tend to share a compute unit, then have a constant amount of work.
+    const int w = blockIdx.x / ny, longs = (a.n_tiles + 1) / 2;
+    const int tile = w < longs ? a.n_tiles - 1 - w : w - longs;
+    const int kvh = y / hblks, hin = (y % hblks) * 4 + wave;
+    const bool head_ok = hin < G;  // a wave without a head still fetches its share of the keys and values
+    const int head = kvh * G + (head_ok ? hin : 0);
+    const int4 info = *reinterpret_cast<const int4*>(a.tiles + (size_t)tile * TILE_INTS);
+    const int b = info.x, t0 = info.y, q0 = info.z, n = info.w;
+    const int kv_len = a.tiles[(size_t)tile * TILE_INTS + 4];
+    const int* table = a.block_table + (size_t)b * a.table_stride;
+    constexpr int psh = __builtin_ctz(PS), pmask = PS - 1;
+
+    bool col_ok[2];
+    int pos[2], lo[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int ti = t0 + u * 16 + c;
+      col_ok[u] = ti < n && head_ok;
+      pos[u] = col_ok[u] ? kv_len - n + ti : -1;
+      lo[u] = (col_ok[u] && a.window > 0) ? max(0, pos[u] - a.window + 1) : 0;
+    }
+    // what the tile's tokens see, from the descriptor alone: the same in every wave
+    const int first_pos = kv_len - n + t0, last_pos = kv_len - n + min(t0 + 31, n - 1);
+    const int whi = last_pos + 1;                                                   // keys [wlo, whi) are seen by some token
+    const int wlo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
+    const int full_hi = first_pos;                                                  // keys <= full_hi are seen by every token
+    const int full_lo = a.window > 0 ? max(0, last_pos - a.window + 1) : 0;         // ... if they are >= full_lo
+    const int kb0 = wlo / 32, kb1 = (whi + 31) / 32;
+
+    bf16x8 qw[2][NQ];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int ti = t0 + u * 16 + c;
+      const bf16_t* qrow = a.q + (size_t)(q0 + (col_ok[u] ? ti : 0)) * a.q_stride + head * HD;
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) {
+        qw[u][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32 + g * 8);
+        if (!col_ok[u]) qw[u][i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+    f32x4 o[2][DT];
+    float m[2], lsum[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      m[u] = -INFINITY;
+      lsum[u] = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[u][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // This thread's pieces of a block: piece r of the keys is 8 channels of one key, piece r of the values 8 keys of
+    // one channel.
+    int k_key[PER_THREAD], k_off[PER_THREAD], k_lds[PER_THREAD];
+    int v_kq[PER_THREAD], v_ch[PER_THREAD], v_lds[PER_THREAD];
+    bool mine[PER_THREAD];
+#pragma unroll
+    for (int r = 0; r < PER_THREAD; ++r) {
+      const int qi = tid + 256 * r;
+      mine[r] = qi < CHUNKS;
+      const int q = mine[r] ? qi : 0;
+      const int key = q / (HD / 8), piece = q % (HD / 8);
+      k_key[r] = key;
+      k_off[r] = piece * 8;
+      k_lds[r] = (16 * ((key & 7) >> 2) + 4 * (key >> 3) + (key & 3)) * KROW + piece * 8;
+      const int pg = q / (CPR * HD), rem = q % (CPR * HD);
+      v_ch[r] = rem / CPR;
+      v_kq[r] = pg * CPR + rem % CPR;
+      v_lds[r] = v_ch[r] * VROW + v_kq[r] * 8;
+    }
+    const int vlo = wlo & ~7, vhi = (whi - 1) & ~7;
+    const size_t k_head = ((size_t)kvh * HD) << psh, kv_page = ((size_t)a.kv_heads * HD) << psh;  // elements
+    // A block that lies wholly inside [wlo, whi) and pages that divide a block: page slots and offsets inside a page
+    // are the same in every block, up to the block's first slot.
+    constexpr bool EVEN = PS <= 32;
+    constexpr int PPB = EVEN ? 32 / PS : 1;  // pages per block
+    int k_slot[PER_THREAD], v_slot[PER_THREAD], k_const[PER_THREAD], v_const[PER_THREAD];
+#pragma unroll
+    for (int r = 0; r < PER_THREAD; ++r) {
+      k_slot[r] = k_key[r] >> psh;
+      v_slot[r] = (v_kq[r] * 8) >> psh;
+      k_const[r] = (int)k_head + (k_key[r] & pmask) * HD + k_off[r];
+      v_const[r] = (int)k_head + (v_ch[r] << psh) + ((v_kq[r] * 8) & pmask);
+    }
+    auto inside = [&](int kb) { return EVEN && kb * 32 >= wlo && kb * 32 + 31 < whi; };
+    int kp[PER_THREAD], vp[PER_THREAD];
+    bf16x8 kst[PER_THREAD], vst[PER_THREAD];
+    // Otherwise addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
+    auto fetch_pages = [&](int kb) {
+      if (inside(kb)) {
+        const int* row = table + kb * PPB;
+#pragma unroll
+        for (int r = 0; r < PER_THREAD; ++r) {
+          kp[r] = row[k_slot[r]];
+          vp[r] = row[v_slot[r]];
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < PER_THREAD; ++r) {
+          kp[r] = table[min(max(kb * 32 + k_key[r], wlo), whi - 1) >> psh];
+          vp[r] = table[min(max(kb * 32 + v_kq[r] * 8, vlo), vhi) >> psh];
+        }
+      }
+    };
+    auto fetch = [&](int kb) {
+      if (inside(kb)) {
+#pragma unroll
+        for (int r = 0; r < PER_THREAD; ++r) {
+          kst[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp[r] * kv_page + k_const[r]);
+          vst[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp[r] * kv_page + v_const[r]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < PER_THREAD; ++r) {
+          const int key = min(max(kb * 32 + k_key[r], wlo), whi - 1);
+          kst[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp[r] * kv_page + k_head + (size_t)(key & pmask) * HD + k_off[r]);
+          const int key8 = min(max(kb * 32 + v_kq[r] * 8, vlo), vhi);
+          vst[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp[r] * kv_page + k_head + ((size_t)v_ch[r] << psh) + (key8 & pmask));
+        }
+      }
+    };
+    auto put = [&](int buf) {
+#pragma unroll
+      for (int r = 0; r < PER_THREAD; ++r)
+        if (mine[r]) {
+          *reinterpret_cast<bf16x8*>(&lk[buf][k_lds[r]]) = kst[r];
+          *reinterpret_cast<bf16x8*>(&lv[buf][v_lds[r]]) = vst[r];
+        }
+    };
+
+    auto block = [&](int buf, int kb) {
+      const int key_base = kb * 32;
+      f32x4 s[2][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        bf16x8 kf[NQ];
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) kf[i] = *reinterpret_cast<const bf16x8*>(&lk[buf][(16 * t + c) * KROW + 32 * i + 8 * g]);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[i], qw[u][i], acc, 0, 0, 0);
+          s[u][t] = acc;
+        }
+      }
+      // s[u][t][j] is key key_base + 8 g + 4 t + j of column c
+      const bool full = key_base + 31 <= full_hi && key_base >= full_lo;  // no masks needed (uniform over the workgroup)
+      bf16x8 pf[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        float mx = -INFINITY;
+        if (full) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][t][j]);
+        } else {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int key = key_base + g * 8 + t * 4 + j;
+              const float v = (key >= lo[u] && key <= pos[u]) ? s[u][t][j] : -INFINITY;
+              s[u][t][j] = v;
+              mx = fmaxf(mx, v);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        // m[u] is the running maximum of the raw scores (the scale is positive); p = 2^((s - m) scale log2 e)
+        const float m_new = fmaxf(m[u], mx);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const bool moved = m_new != m[u];
+        const float alpha = fast_exp2((m[u] - m_safe) * a.scale_log2);
+        const float shift = -m_safe * a.scale_log2;
+        m[u] = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p = fast_exp2(fmaf(s[u][t][j], a.scale_log2, shift));
+            psum += p;
+            pf[u][t * 4 + j] = (bf16_t)p;
+          }
+        if (__any(moved)) {  // the maximum settles early in long rows; rescaling is skipped from then on
+          lsum[u] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[u][dt][j] *= alpha;
+        }
+        lsum[u] += psum;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
+      }
+    };
+
+    if (kb0 < kb1) {
+      fetch_pages(kb0);
+      fetch(kb0);
+      if (kb0 + 1 < kb1) fetch_pages(kb0 + 1);
+      put(0);
+    }
+    __syncthreads();
+    for (int kb = kb0; kb < kb1; ++kb) {
+      const int buf = (kb - kb0) & 1;
+      const bool more = kb + 1 < kb1;
+      if (more) {
+        fetch(kb + 1);
+        if (kb + 2 < kb1) fetch_pages(kb + 2);
+      }
+      if (head_ok) block(buf, kb);
+      if (more) put(buf ^ 1);
+      __syncthreads();
+    }
+
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      lsum[u] += __shfl_xor(lsum[u], 16, 64);
+      lsum[u] += __shfl_xor(lsum[u], 32, 64);
+      if (!col_ok[u]) continue;
+      const size_t col = (size_t)(q0 + t0 + u * 16 + c) * a.heads + head;
+      const float inv = 1.f / lsum[u];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {  // o[u][dt][j] is channel 16 dt + 4 g + j of column c
+        bf16x4 r = {(bf16_t)(o[u][dt][0] * inv), (bf16_t)(o[u][dt][1] * inv), (bf16_t)(o[u][dt][2] * inv), (bf16_t)(o[u][dt][3] * inv)};
+        *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
       }
     }
   }
@@ -445,7 +747,11 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);
   const long blocks = coop ? items : (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
-  if (qt == 2)
+  if (qt == 2 && SHARED_OK) {
+    const long wgs = (long)n_tiles * kv_heads * ((G + 3) / 4);
+    if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
+    attn_prefill_kernel<<<(unsigned)wgs, 256, 0, stream>>>(a);
+  } else if (qt == 2)
     attn_mfma_kernel<2, false, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
   else if (coop)
     attn_mfma_kernel<1, true, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
