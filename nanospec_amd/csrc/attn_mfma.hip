@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Prompt portions when the head size is a multiple of 32 and a page holds 8 tokens or more: a workgroup owns 32 tokens
+// Prompt portions when the head size is a multiple of 32 up to 128 and a page holds 8 tokens or more: a workgroup owns 32 tokens
 // of up to four query heads of one key/value head, one head per wave.  The four waves need the same keys and values,
 // so each block of 32 keys is fetched once per workgroup, a quarter by each wave, and handed round through LDS;
 // the next block is on its way from memory (and its page ids one block further ahead) while this one is used.
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 //   values in LDS: [channel][32 keys], as the pages hold them
 // Rows are padded by 16 bytes, which spreads the 16 rows of one load over all banks.
 // ------------------------------------------------------------------------------------------------
-constexpr bool SHARED_OK = WIDE && PS >= 8;
+constexpr bool SHARED_OK = WIDE && PS >= 8 && HD <= 128;  // larger heads do not fit two waves' registers per SIMD
 constexpr int KROW = HD + 8;               // elements of a key's row in LDS
 constexpr int VROW = 32 + 8;               // elements of a channel's row in LDS
 constexpr int CHUNKS = 32 * HD / 8;        // 16-byte pieces of a block's keys; as many of its values
