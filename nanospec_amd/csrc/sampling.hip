@@ -39,21 +39,39 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
   const int r = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (size_t)r * row_stride;
 
-  // arg-max of the raw logits (lowest index among equals) and their log-sum-exp
-  float best = -INFINITY;
+  // arg-max of the raw logits (lowest index among equals) and their log-sum-exp, in one pass: every thread keeps the
+  // sum of exp(z - its own maximum so far)
+  float best = -INFINITY, se = 0.f;
   int best_i = 0x7fffffff;
-  for (int i = tid; i < vocab; i += SP_THREADS) {
-    const float v = z[i];
-    if (v > best) { best = v; best_i = i; }
+  auto take = [&](float v, int i) {
+    if (v > best) {
+      se = se * expf(best - v) + 1.f;  // best = -inf: se is still 0
+      best = v;
+      best_i = i;
+    } else if (v > -INFINITY) {
+      se += expf(v - best);
+    }
+  };
+  if ((((uintptr_t)z) & 15) == 0) {
+    const int n4 = vocab >> 2;
+    const float4* z4 = reinterpret_cast<const float4*>(z);
+    for (int i = tid; i < n4; i += SP_THREADS) {
+      const float4 v = z4[i];
+      take(v.x, 4 * i);
+      take(v.y, 4 * i + 1);
+      take(v.z, 4 * i + 2);
+      take(v.w, 4 * i + 3);
+    }
+    for (int i = 4 * n4 + tid; i < vocab; i += SP_THREADS) take(z[i], i);
+  } else {
+    for (int i = tid; i < vocab; i += SP_THREADS) take(z[i], i);
   }
   const float zmax = block_max(best, scratch);
   if (tid == 0) s_idx = 0x7fffffff;
   __syncthreads();
   if (best == zmax) atomicMin(&s_idx, best_i);
-  float se = 0.f;
-  for (int i = tid; i < vocab; i += SP_THREADS) se += expf(z[i] - zmax);
-  const float lse = zmax + logf(block_sum(se, scratch));  // barriers inside publish s_idx
-  const int amax = s_idx;
+  const float lse = zmax + logf(block_sum(best > -INFINITY ? se * expf(best - zmax) : 0.f, scratch));  // barriers inside publish s_idx
+  const int amax = s_idx < vocab ? s_idx : 0;  // a row without a single comparable value (all NaN or -inf) names token 0
   const float T = temperature[r];
   if (T <= 0.f) {
     if (tid == 0) {
@@ -127,6 +145,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
     if (last_kept >= 0) atomicMax(&s_idx, last_kept);
     __syncthreads();
     tok = s_idx;
+    if (tok < 0) tok = amax;  // nothing stayed (a row of NaN)
   }
   if (tid == 0) {
     out_tok[r] = tok;
