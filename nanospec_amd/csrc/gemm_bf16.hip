@@ -1,16 +1,18 @@
 // bfloat16 matrix products on the matrix cores for few rows (decode and short portions):
 //   out[M, N] = x[M, K] . w[N, K]^T,  M <= 64,  32-bit accumulation,  K a multiple of 8.
 //
-// The work is the streaming of w, read exactly once: a workgroup owns 16 rows of w, its waves split
-// K among themselves and each streams its share of those rows straight from memory into the A
-// operand of v_mfma_f32_16x16x32_bf16 (lane = row r + 16 g holds 8 consecutive k of row r); x is
-// the B operand (lane = token m + 16 g).  Which k sits in which of the instruction's 32 slots is
-// free as long as both operands agree, so lane group g takes the k range [128 s + 32 g, +32) of
-// super-step s: 64 contiguous bytes per lane and 256 per row and step.  Partial sums of the waves
-// meet in LDS and are added in wave order, so the result does not depend on timing.
+// The work is the streaming of w, read exactly once, from a layout made at load time ("tiled") in which every
+// load of a wave is one contiguous kilobyte:
+//   wt[row tile rt][k tile kt][i = 0..3][lane = 16 g + r][e = 0..7] = w[16 rt + r][128 kt + 32 g + 8 i + e]
+// rows padded to a multiple of 16 and k to a multiple of 128 with zeros.  A workgroup owns one row tile; its waves
+// take the k tiles in turn (wave v takes kt = v, v + WAVES, ...), so the workgroup as a whole walks through contiguous
+// memory, and each streams its share straight into the A operand of v_mfma_f32_16x16x32_bf16 (lane = row r + 16 g
+// holds 8 consecutive k of row r); x is the B operand (lane = token m + 16 g), pieces of x beyond K are zero.  Which k
+// sits in which of the instruction's 32 slots is free as long as both operands agree.  Partial sums of the waves meet
+// in LDS and are added in wave order, so the result does not depend on timing.
 //
-// Epilogues: plain store (bfloat16 or 32-bit) or silu(gate) * up with a second weight matrix read in
-// the same pass (reference: model/llama.py:195).
+// Epilogues: plain store (bfloat16 or 32-bit); silu(gate) * up with a second weight matrix read in the same pass
+// (reference: model/llama.py:195); rotation and cache write for the stacked q/k/v matrix.
 // (reference for the products themselves: the nn.Linear calls of model/llama.py:175,184,195,286)
 #include "common.h"
 
@@ -38,126 +40,6 @@ struct RopeKvParams {
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
-template <int MT, int WAVES, int EPI, typename OutT>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(OutT* __restrict__ out, const bf16_t* __restrict__ x,
-                                                                  const bf16_t* __restrict__ w,
-                                                                  const bf16_t* __restrict__ w2, int M, int N, int K,
-                                                                  int x_stride, int out_stride) {
-  constexpr int NACC = EPI == EPI_SILU_MUL ? 2 : 1;
-  __shared__ float red[WAVES][NACC * MT][256];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int nrow = min(n0 + r, N - 1);
-  const bf16_t* wrow = w + (size_t)nrow * K;
-  const bf16_t* w2row = EPI == EPI_SILU_MUL ? w2 + (size_t)nrow * K : nullptr;
-  const bf16_t* xrow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + (size_t)min(mt * 16 + r, M - 1) * x_stride;
-
-  const int steps = (K + 127) / 128;
-  const int per = (steps + WAVES - 1) / WAVES;
-  const int ks0 = wave * per * 128;
-  const int ks1 = min(K, ks0 + per * 128);
-  const int n_full = ks1 > ks0 ? (ks1 - ks0) / 128 : 0;  // super-steps with all 128 k inside K
-
-  f32x4 acc[NACC][MT];
-#pragma unroll
-  for (int a = 0; a < NACC; ++a)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[a][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  // One super-step of operands: 4 fragments of w (and w2) and 4 per token tile of x.
-  struct Stage {
-    bf16x8 wf[NACC][4], xf[MT][4];
-  };
-  auto load = [&](Stage& st, int ks) {
-    const int kk = ks + g * 32;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      st.wf[0][i] = load8(wrow + kk + i * 8);
-      if (EPI == EPI_SILU_MUL) st.wf[NACC - 1][i] = load8(w2row + kk + i * 8);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) st.xf[mt][i] = load8(xrow[mt] + kk + i * 8);
-    }
-  };
-  auto mma = [&](const Stage& st) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int a = 0; a < NACC; ++a)
-          acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.wf[a][i], st.xf[mt][i], acc[a][mt], 0, 0, 0);
-  };
-
-  // Full super-steps, two in flight: the loads of the next one are issued before the products of this one.
-  Stage s0, s1;
-  int ks = ks0;
-  if (n_full > 0) load(s0, ks);
-  int left = n_full;
-  while (left >= 2) {
-    load(s1, ks + 128);
-    mma(s0);
-    if (left > 2) load(s0, ks + 256);
-    mma(s1);
-    ks += 256;
-    left -= 2;
-  }
-  if (left == 1) {
-    mma(s0);
-    ks += 128;
-  }
-  // The ragged end of K: 8-element pieces beyond K are zero.
-  if (ks < ks1) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int kk = ks + g * 32 + i * 8;
-      const bool ok = kk < K;
-      s0.wf[0][i] = ok ? load8(wrow + kk) : zero;
-      if (EPI == EPI_SILU_MUL) s0.wf[NACC - 1][i] = ok ? load8(w2row + kk) : zero;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) s0.xf[mt][i] = ok ? load8(xrow[mt] + kk) : zero;
-    }
-    mma(s0);
-  }
-
-  // acc[a][mt][j] is the sum for w row n0 + 4 g + j and token 16 mt + r.
-#pragma unroll
-  for (int a = 0; a < NACC; ++a)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) red[wave][a * MT + mt][lane * 4 + j] = acc[a][mt][j];
-  __syncthreads();
-  for (int e = threadIdx.x; e < MT * 256; e += WAVES * 64) {
-    const int mt = e >> 8, le = e & 255;
-    const int l = le >> 2, j = le & 3;
-    const int n = n0 + (l >> 4) * 4 + j, m = mt * 16 + (l & 15);
-    if (n >= N || m >= M) continue;
-    float s = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) s += red[wv][mt][le];
-    if (EPI == EPI_SILU_MUL) {
-      float u = 0.f;
-#pragma unroll
-      for (int wv = 0; wv < WAVES; ++wv) u += red[wv][MT + mt][le];
-      s = s / (1.f + expf(-s)) * u;
-    }
-    out[(size_t)m * out_stride + n] = (OutT)s;
-  }
-}
-
-
-// ------------------------------------------------------------------------------------------------
-// The same product from weights that were re-laid at load time into the order in which the matrix
-// instruction wants them ("tiled" layout), so that every load of a wave is one contiguous kilobyte:
-//   wt[row tile rt][k tile kt][i = 0..3][lane = 16 g + r][e = 0..7] = w[16 rt + r][128 kt + 32 g + 8 i + e]
-// rows padded to a multiple of 16 and k to a multiple of 128 with zeros.  A workgroup owns one row tile;
-// its waves take the k tiles in turn (wave v takes kt = v, v + WAVES, ...), so the workgroup as a whole
-// walks through contiguous memory.  x is read as before; pieces of x beyond K are zero.
-// ------------------------------------------------------------------------------------------------
 template <int MT, int WAVES, int EPI, typename OutT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict__ out, const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ wt,
@@ -351,44 +233,6 @@ static int tiled_dispatch(void* out, const void* x, const void* wt, const void* 
     NS_TILED(4)
   }
 #undef NS_TILED
-  return NS_ERR_BAD_ARG;
-}
-
-template <int MT, int WAVES>
-static int launch_skinny(void* out, const void* x, const void* w, const void* w2, int M, int N, int K, int x_stride,
-                         int out_stride, int epi, int out_f32, hipStream_t stream) {
-  const int grid = (N + 15) / 16;
-  const bf16_t* xb = (const bf16_t*)x;
-  const bf16_t* wb = (const bf16_t*)w;
-  const bf16_t* w2b = (const bf16_t*)w2;
-  if (epi == EPI_SILU_MUL) {
-    if (out_f32) return NS_ERR_UNSUPPORTED;
-    gemm_skinny_kernel<MT, WAVES, EPI_SILU_MUL, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, w2b, M, N, K, x_stride, out_stride);
-  } else if (out_f32) {
-    gemm_skinny_kernel<MT, WAVES, EPI_STORE, float><<<grid, WAVES * 64, 0, stream>>>((float*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride);
-  } else {
-    gemm_skinny_kernel<MT, WAVES, EPI_STORE, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride);
-  }
-  return ns_launch_status();
-}
-
-// epi: 0 = store, 1 = silu(x.w^T) * (x.w2^T).  waves: 4 or 8 waves per workgroup share K.
-extern "C" int ns_gemm_skinny_bf16(void* out, const void* x, const void* w, const void* w2, int M, int N, int K,
-                                   int x_stride, int out_stride, int epi, int out_f32, int waves, hipStream_t stream) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
-  if (epi == EPI_SILU_MUL && !w2) return NS_ERR_BAD_ARG;
-  const int mt = (M + 15) / 16;
-#define NS_SKINNY(MTV)                                                                                              \
-  case MTV:                                                                                                         \
-    return waves == 8 ? launch_skinny<MTV, 8>(out, x, w, w2, M, N, K, x_stride, out_stride, epi, out_f32, stream)   \
-                      : launch_skinny<MTV, 4>(out, x, w, w2, M, N, K, x_stride, out_stride, epi, out_f32, stream);
-  switch (mt) {
-    NS_SKINNY(1)
-    NS_SKINNY(2)
-    NS_SKINNY(3)
-    NS_SKINNY(4)
-  }
-#undef NS_SKINNY
   return NS_ERR_BAD_ARG;
 }
 

@@ -185,30 +185,6 @@ def linear_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = 
 SKINNY_MAX_ROWS = 64
 
 
-def skinny_takes(x: torch.Tensor, w: torch.Tensor) -> bool:
-    return (x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and w.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
-            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-
-
-def linear_skinny(x: torch.Tensor, w: torch.Tensor, w2: torch.Tensor | None = None, out: torch.Tensor | None = None,
-                  out_f32: bool = False, waves: int = 0) -> torch.Tensor:
-    """bfloat16 x @ w.T for at most 64 rows on the matrix cores; with ``w2``: silu(x @ w.T) * (x @ w2.T)."""
-    out = _check_linear(x, w, out, out_f32)
-    if not skinny_takes(x, w):
-        raise KernelRefused(f"linear_skinny takes bfloat16, at most {SKINNY_MAX_ROWS} rows and an inner size that is a multiple of 8; "
-                            f"got x {tuple(x.shape)} {x.dtype}")
-    if w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous() or w2.data_ptr() % 16):
-        raise KernelRefused("linear_skinny: w2 must match w")
-    m, k = x.shape
-    if waves == 0:
-        # enough waves in flight to keep the memory system busy: 8 waves share K when a launch has few workgroups
-        waves = 8 if (w.shape[0] + 15) // 16 < 1024 and k >= 2048 else 4
-    _check(build.core().ns_gemm_skinny_bf16(_ptr(out), _ptr(x), _ptr(w), _ptr(w2), c_int(m), c_int(w.shape[0]), c_int(k),
-                                            c_int(x.stride(0)), c_int(out.stride(0)), c_int(1 if w2 is not None else 0),
-                                            c_int(1 if out_f32 else 0), c_int(waves), _stream()), "linear_skinny")
-    return out
-
-
 class TiledWeight:
     """A bfloat16 weight matrix [N, K] re-laid for the streaming matrix-core kernel:
     wt[rt][kt][i][lane = 16 g + r][e] = w[16 rt + r][128 kt + 32 g + 8 i + e], rows padded to a multiple of 16 and

@@ -74,27 +74,6 @@ def test_linear_generic(dtype, m, n, k):
     assert torch.equal(ops.linear_generic(x[:1].contiguous(), w, out_f32=True), out[:1])
 
 
-@pytest.mark.parametrize("m", [1, 3, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064)])
-def test_linear_skinny(m, n, k):
-    ops = _ops()
-    torch.manual_seed(m + n + k)
-    x = torch.randn(m, k, dtype=torch.bfloat16, device=DEV)
-    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
-    ref = x.cpu().float() @ w.cpu().float().T
-    for waves in (4, 8):
-        out = ops.linear_skinny(x, w, out_f32=True, waves=waves)
-        torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
-    out = ops.linear_skinny(x, w)
-    assert ulps_of_row_max(out.cpu(), ref).max() <= 1.0
-    # fused silu(gate) * up
-    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
-    g, u = ref, x.cpu().float() @ w2.cpu().float().T
-    act = ops.linear_skinny(x, w, w2=w2)
-    want = g * torch.sigmoid(g) * u
-    assert ulps_of_row_max(act.cpu(), want).max() <= 1.0
-
-
 @pytest.mark.parametrize("m", [1, 7, 16, 33, 64])
 @pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064), (16, 8), (4096, 14336)])
 def test_linear_tiled(m, n, k):
@@ -143,16 +122,20 @@ def test_linear_wide(m, n, k):
         assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0
 
 
-def test_linear_skinny_refuses():
+def test_linear_tiled_refuses():
     ops = _ops()
     from nanospec_amd.kernels import KernelRefused
 
-    x = torch.randn(65, 64, dtype=torch.bfloat16, device=DEV)
     w = torch.randn(16, 64, dtype=torch.bfloat16, device=DEV)
+    wt = ops.TiledWeight(w)
     with pytest.raises(KernelRefused):
-        ops.linear_skinny(x, w)
+        ops.linear_tiled(torch.randn(65, 64, dtype=torch.bfloat16, device=DEV), wt)  # too many rows
     with pytest.raises(KernelRefused):
-        ops.linear_skinny(x[:4, :60], w[:, :60].contiguous())
+        ops.linear_tiled(torch.randn(4, 60, dtype=torch.bfloat16, device=DEV), wt)  # inner size differs
+    with pytest.raises(KernelRefused):
+        ops.linear_tiled(torch.randn(4, 64, dtype=torch.float32, device=DEV), wt)
+    with pytest.raises(KernelRefused):
+        ops.TiledWeight(w.float())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
