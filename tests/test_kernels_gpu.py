@@ -278,6 +278,8 @@ CASES = {
     "append6": ([37], [6]),
     "mixed": ([21, 50, 0], [1, 6, 9]),
     "long": ([300, 0, 511], [1, 70, 1]),
+    # more than 64 pages a request at every page size: the kernels hold 64 page ids at a time
+    "beyond64pages": ([1300, 0], [1, 1100]),
 }
 
 
