@@ -6,7 +6,8 @@
 // whole-row loads, into LDS and read from there by every wave in the layout the matrix instruction wants.  The weights
 // still go from memory straight into registers, each exactly once.  Since 64 rows per workgroup leave too few workgroups
 // to fill the GPU, K is cut into `ksplit` ranges over blockIdx.y; each range writes 32-bit partial sums and a second
-// kernel adds the ranges in order and applies the epilogue (store as bfloat16 or 32-bit, or silu(gate) * up).
+// kernel adds the ranges in order and applies the epilogue (store as bfloat16 or 32-bit, or silu(gate) * up).  With a
+// single range the first kernel applies the epilogue itself and nothing is written twice.
 // (reference for the products: the nn.Linear calls of model/llama.py:175,184,195,286)
 #include "common.h"
 
@@ -18,10 +19,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 // partial[(a * ksplit + s) * M * N + m * N + n]: sum over k range s of matrix a (0: w, 1: w2)
 // NT: 16-row tiles of w per wave (64 NT rows per workgroup); each fragment of x read from LDS serves all of them.
+// direct_out (only with ksplit == 1): the result goes there, as 32-bit if out_f32, else as bfloat16.
 template <int MT, int NACC, int NT>
 __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ partial, const bf16_t* __restrict__ x,
                                                         const bf16_t* __restrict__ wt, const bf16_t* __restrict__ wt2,
-                                                        int M, int N, int K, int x_stride, int ksplit) {
+                                                        int M, int N, int K, int x_stride, int ksplit,
+                                                        void* __restrict__ direct_out, int out_stride, int out_f32) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][WIDE_XROW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -113,6 +116,27 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
 
   if (!has_rows) return;
   // acc[a][t][mt][j] is the sum for w row 16 (rt + t) + 4 g + j and token 16 mt + r
+  if (direct_out) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + r, n = (rt + t) * 16 + g * 4;
+        if (m >= M || !tile_ok[t]) continue;
+        f32x4 v = acc[0][t][mt];
+        if (NACC == 2) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = v[j] / (1.f + expf(-v[j])) * acc[NACC - 1][t][mt][j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < N) {
+            if (out_f32) ((float*)direct_out)[(size_t)m * out_stride + n + j] = v[j];
+            else ((bf16_t*)direct_out)[(size_t)m * out_stride + n + j] = (bf16_t)v[j];
+          }
+      }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < NACC; ++a)
 #pragma unroll
@@ -151,37 +175,38 @@ __global__ void gemm_wide_reduce_kernel(OutT* __restrict__ out, const float* __r
 
 template <int MT>
 static int launch_wide(float* partial, const bf16_t* x, const bf16_t* wt, const bf16_t* wt2, int M, int N, int K, int x_stride,
-                       int ksplit, int nt, hipStream_t stream) {
+                       int ksplit, int nt, void* direct_out, int out_stride, int out_f32, hipStream_t stream) {
   const int row_tiles = (N + 15) / 16;
   dim3 grid((row_tiles + 4 * nt - 1) / (4 * nt), ksplit);
   if (wt2 && nt == 2)
-    gemm_wide_kernel<MT, 2, 2><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit);
+    gemm_wide_kernel<MT, 2, 2><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
   else if (wt2)
-    gemm_wide_kernel<MT, 2, 1><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit);
+    gemm_wide_kernel<MT, 2, 1><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
   else if (nt == 2)
-    gemm_wide_kernel<MT, 1, 2><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit);
+    gemm_wide_kernel<MT, 1, 2><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
   else
-    gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit);
+    gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
   return ns_launch_status();
 }
 
-// workspace: (wt2 ? 2 : 1) * ksplit * M * N floats.  epi 0: store; 1: silu(x.w^T) * (x.w2^T).
+// workspace: (wt2 ? 2 : 1) * ksplit * M * N floats (unused with ksplit == 1).  epi 0: store; 1: silu(x.w^T) * (x.w2^T).
 extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
                                  int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, hipStream_t stream) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N || !workspace) return NS_ERR_BAD_ARG;
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
   if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
   const int KT = (K + 127) / 128;
-  if (ksplit < 1 || ksplit > KT || ksplit > 65535 || (nt != 1 && nt != 2)) return NS_ERR_BAD_ARG;
+  if (ksplit < 1 || ksplit > KT || ksplit > 65535 || (nt != 1 && nt != 2) || (ksplit > 1 && !workspace)) return NS_ERR_BAD_ARG;
   const int mt = (M + 15) / 16;
   float* part = (float*)workspace;
+  void* direct = ksplit == 1 ? out : nullptr;
   int st;
   switch (mt) {
-    case 1: st = launch_wide<1>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
-    case 2: st = launch_wide<2>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
-    case 3: st = launch_wide<3>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
-    default: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, stream); break;
+    case 1: st = launch_wide<1>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
+    case 2: st = launch_wide<2>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
+    case 3: st = launch_wide<3>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
+    default: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
   }
-  if (st != NS_OK) return st;
+  if (st != NS_OK || direct) return st;
   const size_t total = (size_t)M * N;
   const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
   if (epi == 1)

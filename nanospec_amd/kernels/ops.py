@@ -259,7 +259,7 @@ def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, 
                 out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0) -> torch.Tensor:
     """bfloat16 x @ w.T for up to 64 rows from a tiled weight, with the tile of x shared through LDS by the four waves of
     a workgroup and K cut into ``ksplit`` ranges that a second kernel adds up; with ``w2``: silu(x @ w.T) * (x @ w2.T).
-    ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values."""
+    ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values (none for a single range)."""
     _gpu(x, out, workspace)
     if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k):
         raise KernelRefused(f"linear_wide takes bfloat16 x [rows <= {SKINNY_MAX_ROWS}, {w.k}] with an inner size that is a "
@@ -274,12 +274,12 @@ def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, 
         raise KernelRefused("linear_wide: w2 must match w and the gated result is bfloat16")
     plan = wide_plan(w.n, w.k)
     ksplit, nt = ksplit or plan[0], nt or plan[1]
-    need = (2 if w2 is not None else 1) * ksplit * m * w.n
-    if workspace is None:
+    need = (2 if w2 is not None else 1) * ksplit * m * w.n if ksplit > 1 else 0  # a single range writes the result itself
+    if workspace is None and need:
         workspace = torch.empty(need, dtype=torch.float32, device=x.device)
-    if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+    if need and (workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous()):
         raise KernelRefused("linear_wide: workspace too small")
-    _check(build.core().ns_gemm_wide_bf16(_ptr(out), _ptr(workspace), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None),
+    _check(build.core().ns_gemm_wide_bf16(_ptr(out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None),
                                           c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
                                           c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), _stream()),
            "linear_wide")

@@ -44,7 +44,7 @@ class LinearWeight:
             return ops.linear_tiled(x, self.tiled, out=out, out_f32=out_f32)
         if self.tiled is not None and m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None or self.n <= WIDE_MAX_N):
             ksplit, nt = ops.wide_plan(self.n, self.k)
-            ws = arena.take((ksplit * m * self.n,), torch.float32) if arena is not None else None
+            ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
             return ops.linear_wide(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
         if self.plain is not None and (not out_f32 or self.tiled is None):
             if out_f32:
@@ -53,7 +53,7 @@ class LinearWeight:
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
         ksplit, nt = ops.wide_plan(self.n, self.k)
-        ws = arena.take((ksplit * ops.SKINNY_MAX_ROWS * self.n,), torch.float32) if arena is not None else None
+        ws = arena.take((ksplit * ops.SKINNY_MAX_ROWS * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
         for s in range(0, m, ops.SKINNY_MAX_ROWS):
             e = min(m, s + ops.SKINNY_MAX_ROWS)
             if e - s <= STREAM_ROWS:
@@ -78,13 +78,12 @@ class GatedWeights:
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
-        if fast and self.stacked is None:
-            # (with the plain layout at hand the library's product plus the activation kernel is faster from 17 rows on)
-            ksplit, nt = ops.wide_plan(self.inter, self.k)
-            ws = ctx.arena.take((2 * ksplit * min(m, ops.SKINNY_MAX_ROWS) * self.inter,), torch.float32)
+        if fast and (m <= ops.SKINNY_MAX_ROWS or self.stacked is None):
+            # 17 to 64 rows: the second hand-written kernel, one range of K, so that the activation is applied in the same
+            # pass (measured ahead of the library's product plus the activation kernel)
             for s in range(0, m, ops.SKINNY_MAX_ROWS):
                 e = min(m, s + ops.SKINNY_MAX_ROWS)
-                ops.linear_wide(x[s:e], self.tiled[0], w2=self.tiled[1], out=out[s:e], workspace=ws, ksplit=ksplit, nt=nt)
+                ops.linear_wide(x[s:e], self.tiled[0], w2=self.tiled[1], out=out[s:e], ksplit=1, nt=1)
             return out
         gu = ctx.arena.take((m, 2 * self.inter), x.dtype)
         if self.dtype == torch.float32 or self.k % 8:
