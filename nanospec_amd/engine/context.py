@@ -66,8 +66,11 @@ class AttentionPlan:
 class StepContext:
     """Device views of one step's batch plus the arena; handed to every part."""
 
-    def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, fixed_splits: bool = False) -> None:
+    def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, fixed_splits: bool = False,
+                 link_norms: bool = True) -> None:
         self.layout, self.arena = layout, arena
+        # blocks may let the products around an RMS norm do the norm's work (see parts.block.PreNormBlock.forward)
+        self.link_norms = link_norms
         self.n_tokens, self.n_reqs = layout.N, layout.B
         self.max_position, self.max_kv_len = max_position, max_kv_len
         self.fixed_splits = fixed_splits

@@ -59,7 +59,7 @@ class _DecodeGraph:
         return f[0], f[1], f[2], opts[3]
 
     def context(self, runner) -> StepContext:
-        return StepContext(self.layout, self.dev_buf, self.arena, max_position=0, max_kv_len=runner.table_width * runner.page_size,
+        return StepContext(self.layout, self.dev_buf, self.arena, link_norms=runner.link_norms, max_position=0, max_kv_len=runner.table_width * runner.page_size,
                            fixed_splits=True)
 
 
@@ -73,6 +73,7 @@ class ModelRunner:
         self.max_requests = max_requests
         self.stream = torch.cuda.Stream(device=self.device)
         self.arena = Arena(self.device)
+        self.link_norms = True  # see StepContext; set False before the first step to run every norm as a kernel of its own
         n_groups = len(manager.groups)
         # host mirror of every live request's block tables, one row per state slot
         self._tables = [np.full((manager.slots.num_slots, table_width), -1, dtype=np.int32) for _ in range(n_groups)]
@@ -223,7 +224,7 @@ class ModelRunner:
         if n_patch:
             self._apply_patch(self._dev, layout, device_tokens[0], n_patch)
         self.arena.reset()
-        ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv)
+        ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv, link_norms=self.link_norms)
         resid, delta = self.model.forward_hidden(ctx, self.storage.views)
         if not n_want:
             return None

@@ -222,9 +222,33 @@ def tiled_takes(x: torch.Tensor, k: int) -> bool:
             and x.stride(1) == 1 and x.data_ptr() % 16 == 0)
 
 
-def linear_tiled(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
+class PreNormed:
+    """The input of an RMS norm's consumer when the norm has no kernel of its own: ``x`` = r * weight [rows, dim] in bfloat16
+    (r the rows to normalise), and ``ssq`` [rows, parts], float32, whose sum over parts is each row's sum of r^2.  The
+    consumer multiplies its sums by rsqrt(sum / dim + eps): y = w * r / rms(r) is linear in 1/rms(r).  Made by
+    ``linear_resid_norm``; taken by ``linear_tiled`` and ``linear_qkv_rope`` for at most 16 rows."""
+
+    def __init__(self, x: torch.Tensor, ssq: torch.Tensor, dim: int, eps: float) -> None:
+        self.x, self.ssq, self.dim, self.eps = x, ssq, dim, eps
+        self.shape, self.dtype = x.shape, x.dtype
+
+
+def _prenorm_args(pre: "PreNormed | None", m: int, what: str):
+    if pre is None:
+        return c_void_p(None), c_int(0), c_int(0), c_float(0.0)
+    if (pre.ssq.dtype != torch.float32 or pre.ssq.dim() != 2 or pre.ssq.shape[0] != m or not pre.ssq.is_contiguous() or m > 16
+            or not pre.ssq.is_cuda):
+        raise KernelRefused(f"{what}: the sums of squares must be float32 [rows, parts] for at most 16 rows")
+    return _ptr(pre.ssq), c_int(pre.ssq.shape[1]), c_int(pre.dim), c_float(pre.eps)
+
+
+def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
                  out_f32: bool = False, waves: int = 0) -> torch.Tensor:
-    """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T)."""
+    """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T).  ``x`` may be a
+    ``PreNormed`` (at most 16 rows)."""
+    pre = x if isinstance(x, PreNormed) else None
+    if pre is not None:
+        x = pre.x
     _gpu(x, out)
     if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k):
         raise KernelRefused(f"linear_tiled takes bfloat16 x [rows <= {SKINNY_MAX_ROWS}, {w.k}] with an inner size that is a "
@@ -241,9 +265,39 @@ def linear_tiled(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None,
         waves = 8 if w.k >= 8192 or (w.n // 16 < 512 and w.k >= 2048) else 4
     _check(build.core().ns_gemm_tiled_bf16(_ptr(out), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None), c_int(m),
                                            c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
-                                           c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(waves), _stream()),
+                                           c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(waves),
+                                           *_prenorm_args(pre, m, "linear_tiled"), _stream()),
            "linear_tiled")
     return out
+
+
+def linear_resid_norm(x: torch.Tensor, w: TiledWeight, resid: torch.Tensor, next_weight: torch.Tensor, eps: float,
+                      x_next: torch.Tensor | None = None, ssq: torch.Tensor | None = None, waves: int = 0) -> PreNormed:
+    """A block's contribution to the residual stream, for at most 16 rows: resid += x @ w.T in place (the product and
+    the sum rounded to bfloat16 in turn, as separate kernels would), and what the RMS norm that follows needs from it:
+    -> PreNormed(resid * next_weight, per-workgroup sums of resid^2)."""
+    _gpu(x, resid, next_weight, x_next, ssq)
+    m = x.shape[0]
+    if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k) or m > 16:
+        raise KernelRefused(f"linear_resid_norm takes at most 16 bfloat16 rows of {w.k} values; got {tuple(x.shape)} {x.dtype}")
+    if resid.shape != (m, w.n) or resid.dtype != torch.bfloat16 or resid.stride(1) != 1:
+        raise KernelRefused("linear_resid_norm: resid must be bfloat16 [rows, out features]")
+    if next_weight.shape != (w.n,) or next_weight.dtype != torch.bfloat16 or not next_weight.is_contiguous():
+        raise KernelRefused("linear_resid_norm: the next norm's weight must be bfloat16 [out features]")
+    parts = -(-w.n // 16)
+    if x_next is None:
+        x_next = torch.empty_like(resid)
+    if ssq is None:
+        ssq = torch.empty((m, parts), dtype=torch.float32, device=x.device)
+    if (x_next.shape != resid.shape or x_next.dtype != resid.dtype or x_next.stride() != resid.stride()
+            or ssq.shape != (m, parts) or ssq.dtype != torch.float32 or not ssq.is_contiguous()):
+        raise KernelRefused("linear_resid_norm: x_next must be laid out like resid, ssq float32 [rows, ceil(out features / 16)]")
+    if waves == 0:
+        waves = 8 if w.k >= 8192 or (w.n // 16 < 512 and w.k >= 2048) else 4
+    _check(build.core().ns_gemm_resid_norm_bf16(_ptr(resid), _ptr(x_next), _ptr(ssq), _ptr(next_weight), _ptr(x), _ptr(w.data),
+                                                c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(resid.stride(0)),
+                                                c_int(waves), _stream()), "linear_resid_norm")
+    return PreNormed(x_next, ssq, w.n, eps)
 
 
 def wide_plan(n: int, k: int) -> tuple[int, int]:
@@ -305,11 +359,15 @@ def qkv_rope_takes(x: torch.Tensor, head_dim: int, rotary_dim: int) -> bool:
     return x.dtype == torch.bfloat16 and x.shape[0] <= 16 and head_dim % 16 == 0 and rotary_dim % 16 == 0
 
 
-def linear_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, positions, token_req, block_table, inv_freq, k_cache,
-                    v_cache, heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True, waves: int = 0) -> None:
+def linear_qkv_rope(x: "torch.Tensor | PreNormed", w: TiledWeight, q_out: torch.Tensor, positions, token_req, block_table, inv_freq,
+                    k_cache, v_cache, heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True,
+                    waves: int = 0) -> None:
     """The stacked q/k/v product of at most 16 tokens with rotation and cache write fused into its epilogue: q goes rotated
     into ``q_out`` [M, >= heads * head_dim], k rotated into its K page slot, v into the transposed V page.  ``w`` is the
-    stacked matrix tiled in ``qkv_rope_row_order``."""
+    stacked matrix tiled in ``qkv_rope_row_order``.  ``x`` may be a ``PreNormed``."""
+    pre = x if isinstance(x, PreNormed) else None
+    if pre is not None:
+        x = pre.x
     _gpu(x, q_out, positions, token_req, block_table, inv_freq, k_cache, v_cache)
     m = x.shape[0]
     if not (tiled_takes(x, w.k) and qkv_rope_takes(x, head_dim, rotary_dim)) or x.shape[1] != w.k:
@@ -331,7 +389,8 @@ def linear_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, positi
                                               c_int(q_out.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
                                               c_int(block_table.stride(0)), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(heads),
                                               c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(page),
-                                              c_int(1 if write_kv else 0), c_int(waves), _stream()), "linear_qkv_rope")
+                                              c_int(1 if write_kv else 0), c_int(waves), *_prenorm_args(pre, m, "linear_qkv_rope"),
+                                              _stream()), "linear_qkv_rope")
 
 
 # ------------------------------------------------------------------------------------------------ attention

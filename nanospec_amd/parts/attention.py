@@ -70,7 +70,12 @@ class Attention:
     def cache_need(self):
         return PagedNeed(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
 
-    def forward(self, ctx, x: torch.Tensor, cache, owns_cache: bool = True, out: torch.Tensor | None = None) -> torch.Tensor:
+    def links_norms(self, rows: int) -> bool:
+        """Whether, for this many rows, ``forward`` takes a ``PreNormed`` input and an ``IntoResidual`` ending."""
+        first = self.wqkv_rope is not None or self.wqkv.links_norms(rows)
+        return rows <= 16 and first and self.wo.links_norms(rows)
+
+    def forward(self, ctx, x, cache, owns_cache: bool = True, out: torch.Tensor | None = None, residual=None):
         s = self.spec
         n = x.shape[0]
         pos = self.position
@@ -78,7 +83,7 @@ class Attention:
             raise ValueError(f"position {ctx.max_position} is beyond the model's {pos.max_positions} positions")
         qkv = ctx.arena.take((n, self.wqkv.n), x.dtype)
         table = ctx.block_tables[cache.group]
-        if self.wqkv_rope is not None and n <= 16 and ops.tiled_takes(x, s.hidden):
+        if self.wqkv_rope is not None and n <= 16 and ops.tiled_takes(x.x if isinstance(x, ops.PreNormed) else x, s.hidden):
             ops.linear_qkv_rope(x, self.wqkv_rope, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v,
                                 s.heads, s.kv_heads, s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         else:
@@ -96,6 +101,8 @@ class Attention:
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)
+        if residual is not None:
+            return self.wo.into_residual(att, residual, arena=ctx.arena)
         return self.wo(att, out=out, arena=ctx.arena)
 
 

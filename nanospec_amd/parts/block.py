@@ -6,7 +6,11 @@ done inside the norm kernel that follows it (the reference's fused form, model/l
 
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from . import registry
+from .linear import IntoResidual
 
 _MIXER_PREFIX = {"attention": "self_attn."}
 _FFN_PREFIX = {"swiglu": "mlp."}
@@ -39,14 +43,44 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def forward(self, ctx, resid, delta, cache, owns_cache, delta_out) -> None:
+    links_blocks = True  # forward takes next_norm and next_sums
+
+    def forward(self, ctx, resid, delta, cache, owns_cache, delta_out, next_norm=None, next_sums=None):
+        """``delta``: what the block before left to be added (a tensor, or None at the start), or a ``PreNormed``: then
+        ``resid`` is already whole and the first norm's input comes ready for a product that ``links_norms``.
+        ``next_norm``: the norm that will read this block's result (the next block's first one), if it
+        ``links_products``; ``next_sums``: float32 [tokens, ceil(width / 16)] that lives as long as the step.
+        -> None, with the block's not yet added output in ``delta_out``; or a ``PreNormed`` for ``next_norm`` (its rows
+        in ``delta_out``, its sums in ``next_sums``), with ``resid`` whole."""
+        n = resid.shape[0]
         mark = ctx.arena.mark()
-        h = self.mixer_norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None,
-                                    out=ctx.arena.take(resid.shape, resid.dtype))
-        a = self.mixer.forward(ctx, h, cache, owns_cache, out=ctx.arena.take(resid.shape, resid.dtype))
-        h2 = self.ffn_norm.forward(ctx, resid=resid, x=a, write_resid=True, out=h)
+        link = getattr(ctx, "link_norms", False) and resid.dtype == torch.bfloat16
+        can = lambda part: link and getattr(part, "links_norms", lambda rows: False)(n)
+        lp = lambda norm: link and norm is not None and getattr(norm, "links_products", False) and norm.weight.dtype == resid.dtype
+
+        # first norm and mixer
+        if isinstance(delta, ops.PreNormed):
+            h = delta if can(self.mixer) else self.mixer_norm.forward(ctx, resid=resid, out=ctx.arena.take(resid.shape, resid.dtype))
+        else:
+            h = self.mixer_norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None,
+                                        out=ctx.arena.take(resid.shape, resid.dtype))
+        if can(self.mixer) and lp(self.ffn_norm):
+            h2 = self.mixer.forward(ctx, h, cache, owns_cache, residual=IntoResidual(resid, self.ffn_norm.weight, self.ffn_norm.spec.eps))
+            if not can(self.ffn):
+                h2 = self.ffn_norm.forward(ctx, resid=resid, out=ctx.arena.take(resid.shape, resid.dtype))
+        else:
+            a = self.mixer.forward(ctx, h, cache, owns_cache, out=ctx.arena.take(resid.shape, resid.dtype))
+            h2 = self.ffn_norm.forward(ctx, resid=resid, x=a, write_resid=True, out=ctx.arena.take(resid.shape, resid.dtype))
+
+        # second norm and feed-forward
+        if can(self.ffn) and lp(next_norm) and next_sums is not None:
+            # what the next block reads must outlive this block's scratch: it goes into delta_out and next_sums
+            pre = self.ffn.forward(ctx, h2, residual=IntoResidual(resid, next_norm.weight, next_norm.spec.eps, delta_out, next_sums))
+            ctx.arena.release(mark)
+            return pre
         self.ffn.forward(ctx, h2, out=delta_out)
         ctx.arena.release(mark)
+        return None
 
 
 registry.register("block", "prenorm", PreNormBlock)

@@ -23,6 +23,18 @@ WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the libr
 #                    32-bit results, which the library does not give); wider products go to the library
 
 
+class IntoResidual:
+    """Asks a part to end in ``resid += output`` (in place) and to hand back what the RMS norm after it needs
+    (``kernels.ops.PreNormed``), instead of returning its output: the part's last product then does the work of the
+    residual sum and of the norm's statistics.  ``next_weight``, ``eps``: that norm's weight and epsilon.  ``x_next``
+    (like resid) and ``ssq`` (float32 [rows, ceil(width / 16)]): where to put them, if they must outlive the step's
+    scratch."""
+
+    def __init__(self, resid: torch.Tensor, next_weight: torch.Tensor, eps: float, x_next: torch.Tensor | None = None,
+                 ssq: torch.Tensor | None = None) -> None:
+        self.resid, self.next_weight, self.eps, self.x_next, self.ssq = resid, next_weight, eps, x_next, ssq
+
+
 class LinearWeight:
     def __init__(self, w: torch.Tensor, keep_plain: bool = True, tiled: bool = True) -> None:
         """``w``: [out, in] on the GPU in the compute dtype.  ``tiled=False``: the caller streams this matrix with a
@@ -33,8 +45,29 @@ class LinearWeight:
         self.tiled = ops.TiledWeight(w) if (fast and tiled) else None
         self.plain = w if (keep_plain or self.tiled is None) else None
 
-    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_f32: bool = False, arena=None) -> torch.Tensor:
-        """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated."""
+    def links_norms(self, rows: int) -> bool:
+        """Whether a product of ``rows`` rows can take a ``PreNormed`` input and can end in the residual stream."""
+        return self.tiled is not None and rows <= STREAM_ROWS
+
+    def into_residual(self, x: torch.Tensor, link: IntoResidual, arena=None) -> "ops.PreNormed":
+        """link.resid += x @ W^T; -> what the norm after it needs."""
+        if not self.links_norms(x.shape[0]):
+            raise ops.KernelRefused("this product cannot end in the residual stream (rows, layout or precision)")
+        m = x.shape[0]
+        x_next, ssq = link.x_next, link.ssq
+        if x_next is None and arena is not None:
+            x_next = arena.take(tuple(link.resid.shape), link.resid.dtype)
+        if ssq is None and arena is not None:
+            ssq = arena.take((m, -(-self.n // 16)), torch.float32)
+        return ops.linear_resid_norm(x, self.tiled, link.resid, link.next_weight, link.eps, x_next=x_next, ssq=ssq)
+
+    def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None) -> torch.Tensor:
+        """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated.
+        ``x`` may be a ``PreNormed`` where ``links_norms`` holds."""
+        if isinstance(x, ops.PreNormed):
+            if not self.links_norms(x.shape[0]):
+                raise ops.KernelRefused("this product cannot take a pre-normed input (rows, layout or precision)")
+            return ops.linear_tiled(x, self.tiled, out=out, out_f32=out_f32)
         if x.dtype != self.dtype:
             raise ops.KernelRefused(f"linear: input is {x.dtype}, the weight {self.dtype}")
         if self.dtype == torch.float32 or self.k % 8 or not ops.tiled_takes(x[:1], self.k):
@@ -73,8 +106,15 @@ class GatedWeights:
         self.tiled = (ops.TiledWeight(gate), ops.TiledWeight(up)) if fast else None
         self.stacked = torch.cat([gate, up]) if (keep_plain or not fast) else None  # [2 I, K] for the two-kernel path
 
-    def __call__(self, ctx, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    def links_norms(self, rows: int) -> bool:
+        return self.tiled is not None and rows <= STREAM_ROWS
+
+    def __call__(self, ctx, x, out: torch.Tensor) -> torch.Tensor:
         m = x.shape[0]
+        if isinstance(x, ops.PreNormed):
+            if not self.links_norms(m):
+                raise ops.KernelRefused("this product cannot take a pre-normed input (rows, layout or precision)")
+            return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)

@@ -75,9 +75,19 @@ class DecoderModel:
         delta = ctx.arena.take((n, self.spec.hidden), self.dtype)
         ops.embed(self.embed, ctx.token_ids, out=resid)
         pending = None
-        for i, call in enumerate(self.spec.run_order):
-            self.layers[call.layer].forward(ctx, resid, pending, caches[i], call.cache_from is None, delta)
-            pending = delta
+        order = self.spec.run_order
+        sums = ctx.arena.take((n, -(-self.spec.hidden // 16)), torch.float32)  # see PreNormBlock.forward
+        for i, call in enumerate(order):
+            layer = self.layers[call.layer]
+            if getattr(layer, "links_blocks", False) and i + 1 < len(order):
+                # the norm that reads this block's result is the next block's first
+                nxt = getattr(self.layers[order[i + 1].layer], "mixer_norm", None)
+                out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta, next_norm=nxt, next_sums=sums)
+            else:
+                if isinstance(pending, ops.PreNormed):
+                    pending = None  # resid is whole already; a block that does not know the hand-over starts from it
+                out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta)
+            pending = out if out is not None else delta
         return resid, pending
 
     def logits(self, ctx, resid, delta, rows: torch.Tensor) -> torch.Tensor:

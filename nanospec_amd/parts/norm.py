@@ -10,6 +10,9 @@ from .registry import register
 
 class RMSNorm:
     graph_safe = True
+    # y = weight * r / rms(r): linear in 1/rms(r), so a product that follows can apply that factor to its sums and a
+    # product that precedes can gather the sum of squares (``parts.linear.IntoResidual``)
+    links_products = True
 
     def __init__(self, spec, name: str) -> None:
         self.spec, self.name = spec, name

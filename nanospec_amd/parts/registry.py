@@ -21,6 +21,12 @@ What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are 
   block        forward(ctx, resid, delta, cache, owns_cache, delta_out) -> None
                                                   resid is updated in place; the not yet added output of
                                                   the block's last part is left in delta_out
+
+Optional, for parts whose products can do the work of the RMS norms around them (``parts.linear.IntoResidual``):
+  norm         links_products = True, weight, spec.eps
+  mixer, ffn   links_norms(rows) -> bool; forward(..., residual=IntoResidual) -> kernels.ops.PreNormed, and x may be
+               a PreNormed
+  block        links_blocks = True; forward(..., next_norm=None, next_sums=None) -> None | PreNormed
 """
 
 from __future__ import annotations

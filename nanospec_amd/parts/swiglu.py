@@ -31,8 +31,14 @@ class SwiGLU:
                                     get(p + "up_proj.weight").to(device=device, dtype=dtype))
         self.down = LinearWeight(get(p + "down_proj.weight").to(device=device, dtype=dtype).contiguous())
 
-    def forward(self, ctx, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    def links_norms(self, rows: int) -> bool:
+        """Whether, for this many rows, ``forward`` takes a ``PreNormed`` input and an ``IntoResidual`` ending."""
+        return self.gate_up.links_norms(rows) and self.down.links_norms(rows)
+
+    def forward(self, ctx, x, out: torch.Tensor | None = None, residual=None):
         act = self.gate_up(ctx, x, out=ctx.arena.take((x.shape[0], self.spec.intermediate), x.dtype))
+        if residual is not None:
+            return self.down.into_residual(act, residual, arena=ctx.arena)
         return self.down(act, out=out, arena=ctx.arena)
 
 

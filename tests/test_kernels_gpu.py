@@ -238,6 +238,72 @@ def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, pa
         assert ulps_of_row_max(v[pg, :, :, off].cpu().reshape(1, -1), v0[t].reshape(1, -1)).max() <= 1.0
 
 
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("hidden,inner", [(136, 264), (4096, 1024), (64, 8)])
+def test_product_that_updates_the_residual_and_feeds_the_next_norm(m, hidden, inner):
+    """resid += x @ W^T with what the following RMS norm needs as by-products, and the products that take them in place of a
+    normalised input, against the plain sum, the plain norm and the plain product."""
+    ops = _ops()
+    torch.manual_seed(m + hidden)
+    eps = 1e-5
+    x = torch.randn(m, inner).to(torch.bfloat16)
+    w = (torch.randn(hidden, inner) / math.sqrt(inner)).to(torch.bfloat16)
+    resid0 = torch.randn(m, hidden).to(torch.bfloat16)
+    w_norm = (1 + 0.2 * torch.randn(hidden)).to(torch.bfloat16)
+    resid = resid0.to(DEV).clone()
+    pre = ops.linear_resid_norm(x.to(DEV), ops.TiledWeight(w.to(DEV)), resid, w_norm.to(DEV), eps)
+    # the sum: product rounded to bfloat16, then added in 32-bit and rounded (reference: model/llama.py:204-208)
+    delta = (x.float() @ w.float().T).to(torch.bfloat16)
+    want = (resid0.float() + delta.float()).to(torch.bfloat16)
+    err = (resid.cpu().float() - want.float()).abs() / want.float().abs().clamp_min(0.25)
+    assert err.max() <= 2.0 ** -6  # a flipped rounding of the product moves the sum by at most two of its last places
+    got = resid.cpu()
+    assert torch.equal(pre.x.cpu(), (got.float() * w_norm.float()).to(torch.bfloat16))
+    assert pre.ssq.shape == (m, -(-hidden // 16))
+    torch.testing.assert_close(pre.ssq.sum(1).cpu(), (got.float() ** 2).sum(-1), rtol=1e-5, atol=1e-6)
+    # consumers: the plain norm of the kernel's own sum, then the plain products
+    normed = pl.rms_norm(got, w_norm, eps)
+    out_n = 152
+    w3 = (torch.randn(out_n, hidden) / math.sqrt(hidden)).to(torch.bfloat16)
+    w4 = (torch.randn(out_n, hidden) / math.sqrt(hidden)).to(torch.bfloat16)
+    ref = normed.float() @ w3.float().T
+    out = ops.linear_tiled(pre, ops.TiledWeight(w3.to(DEV)))
+    assert ulps_of_row_max(out.cpu(), ref).max() <= 2.0
+    out32 = ops.linear_tiled(pre, ops.TiledWeight(w3.to(DEV)), out_f32=True)
+    assert ulps_of_row_max(out32.cpu(), ref).max() <= 1.0
+    up = normed.float() @ w4.float().T
+    act = ops.linear_tiled(pre, ops.TiledWeight(w3.to(DEV)), w2=ops.TiledWeight(w4.to(DEV)))
+    assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * up).max() <= 2.0
+
+
+def test_qkv_product_takes_a_prenormed_input():
+    ops = _ops()
+    torch.manual_seed(3)
+    heads, kvh, hd, rot, page, hidden, eps = 6, 2, 32, 32, 8, 96, 1e-6
+    starts, lens = [3, 0, 9], [5, 1, 2]
+    n = sum(lens)
+    table = scattered_tables([s + l for s, l in zip(starts, lens)], page, 16, seed=2).to(DEV)
+    positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    r = torch.randn(n, hidden).to(torch.bfloat16)
+    w_norm = (1 + 0.2 * torch.randn(hidden)).to(torch.bfloat16)
+    w = (torch.randn((heads + 2 * kvh) * hd, hidden) * 0.3).to(torch.bfloat16)
+    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot))
+    inv = pl.inverse_frequencies(rot, 10000.0, None).to(DEV)
+    ssq = torch.zeros(n, 3)
+    ssq[:, 1] = (r.float() ** 2).sum(-1)  # any split into parts has the same sum
+    pre = ops.PreNormed((r.float() * w_norm.float()).to(torch.bfloat16).to(DEV), ssq.to(DEV), hidden, eps)
+    outs = []
+    for src in (pre, pl.rms_norm(r, w_norm, eps).to(DEV)):
+        q_out = torch.zeros(n, heads * hd, dtype=torch.bfloat16, device=DEV)
+        k, v = make_cache(16, page, kvh, hd, torch.bfloat16)
+        ops.linear_qkv_rope(src, wt, q_out, positions, token_req, table, inv, k, v, heads, kvh, hd, rot)
+        outs.append((q_out.cpu(), k.cpu(), v.cpu()))
+    for a, b in zip(*outs):
+        assert ulps_of_row_max(a.reshape(1, -1), b.reshape(1, -1).float()).max() <= 2.0
+    assert outs[0][1].abs().sum() > 0
+
+
 def fill_cache(k, v, table, lens, page, kvh, hd, dtype, seed=0, scale=1.0):
     """Random keys and values for positions [0, len) of every request, written through the block table.
     -> per request (K [len, kvh, hd], V [len, kvh, hd]) on the CPU."""

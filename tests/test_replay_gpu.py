@@ -61,10 +61,11 @@ def check(ours: torch.Tensor, ref: torch.Tensor, dtype, what: str):
         assert u.max() <= 8, f"{what}: {u.max():.2f} bf16 ulps of the row's largest logit (median {u.median():.2f})"
 
 
-def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True):
+def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, link_norms=True):
     from nanospec_amd.engine.replay import Replayer
 
     rep = Replayer(model, max_tokens, page_size=page, use_graphs=graphs)
+    rep.runner.link_norms = link_norms
     for step, w in zip(steps, where):
         out = rep.step(step["entries"], step["end"])
         if not w:
@@ -132,6 +133,39 @@ def test_graph_and_eager_decode_agree(tiny_folders, name):
     a = replay(model, steps, where, ref, torch.bfloat16, 256, page, graphs=True)
     assert a.runner._graphs, "decode steps did not replay a graph"
     replay(model, steps, where, ref, torch.bfloat16, 256, page, graphs=False)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("schedule", ["tail", "mixed"])
+def test_norms_as_kernels_of_their_own(tiny_folders, name, schedule):
+    """Steps of at most 16 tokens let the products around a norm do its work; here every norm runs as its own kernel,
+    and the steps in which the two ways differ are counted."""
+    from nanospec_amd.kernels import ops
+
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, torch.bfloat16)
+    model = engine_model(folder, name, torch.bfloat16)
+    if schedule == "tail":
+        steps, where = traces.tail_decoded(seqs)
+        max_tokens = 256
+    else:
+        steps, where, max_tokens = traces.mixed(seqs, seed=5)
+    calls = {"linked": 0}
+    real = ops.linear_resid_norm
+
+    def counted(*a, **k):
+        calls["linked"] += 1
+        return real(*a, **k)
+
+    ops.linear_resid_norm = counted
+    try:
+        replay(model, steps, where, ref, torch.bfloat16, max_tokens, page, graphs=False, link_norms=False)
+        assert calls["linked"] == 0
+        replay(model, steps, where, ref, torch.bfloat16, max_tokens, page, graphs=False, link_norms=True)
+        assert calls["linked"] > 0, "no step took the linked path"
+    finally:
+        ops.linear_resid_norm = real
 
 
 def test_trace_run_program(tiny_folders, tmp_path):
