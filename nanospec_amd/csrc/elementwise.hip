@@ -209,6 +209,70 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* _
   }
 }
 
+// The same with 16-byte accesses for q and k (values still go element by element into their transposed page): a
+// thread takes V consecutive channels j.. of the first half and their partners j + rot/2.  For rot/2, hd - rot and
+// the row stride multiples of V elements and 16-byte aligned buffers.
+template <typename T>
+__global__ void rope_kv_vec_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+                                   const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
+                                   const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                   int heads, int kv_heads, int hd, int rot, int page_size, int write_kv) {
+  constexpr int V = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  extern __shared__ float cs[];  // cos[half] | sin[half] of this token's angles
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  T* row = qkv + (size_t)t * row_stride;
+  const int half = rot / 2;
+  const float fpos = (float)pos;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const float ang = fpos * inv_freq[j];
+    cs[j] = cosf(ang);
+    cs[half + j] = sinf(ang);
+  }
+  __syncthreads();
+  const int per_head = half / V;  // vector pairs per head
+  auto turn = [&](const vec_t a, const vec_t b, int j, vec_t& lo, vec_t& hi) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float c = cs[j + e], s = cs[half + j + e];
+      const float x = to_f(a[e]), y = to_f(b[e]);
+      lo[e] = from_f<T>(x * c - y * s);
+      hi[e] = from_f<T>(y * c + x * s);
+    }
+  };
+  for (int u = threadIdx.x; u < heads * per_head; u += blockDim.x) {
+    const int h = u / per_head, j = (u - h * per_head) * V;
+    T* p = row + h * hd + j;
+    vec_t lo, hi;
+    turn(*reinterpret_cast<const vec_t*>(p), *reinterpret_cast<const vec_t*>(p + half), j, lo, hi);
+    *reinterpret_cast<vec_t*>(p) = lo;
+    *reinterpret_cast<vec_t*>(p + half) = hi;
+  }
+  if (!write_kv) return;
+  const int page = block_table[(size_t)token_req[t] * table_stride + pos / page_size];
+  const int off = pos % page_size;
+  const T* krow = row + heads * hd;
+  const T* vrow = krow + kv_heads * hd;
+  T* kdst = k_cache + (size_t)page * kv_heads * page_size * hd + (size_t)off * hd;
+  T* vdst = v_cache + (size_t)page * kv_heads * hd * page_size + off;
+  for (int u = threadIdx.x; u < kv_heads * per_head; u += blockDim.x) {
+    const int h = u / per_head, j = (u - h * per_head) * V;
+    const T* p = krow + h * hd + j;
+    vec_t lo, hi;
+    turn(*reinterpret_cast<const vec_t*>(p), *reinterpret_cast<const vec_t*>(p + half), j, lo, hi);
+    T* d = kdst + (size_t)h * page_size * hd + j;
+    *reinterpret_cast<vec_t*>(d) = lo;
+    *reinterpret_cast<vec_t*>(d + half) = hi;
+  }
+  const int plain = (hd - rot) / V;  // vectors of a head beyond the rotary part
+  for (int u = threadIdx.x; u < kv_heads * plain; u += blockDim.x) {
+    const int h = u / plain, d0 = rot + (u - h * plain) * V;
+    *reinterpret_cast<vec_t*>(kdst + (size_t)h * page_size * hd + d0) = *reinterpret_cast<const vec_t*>(krow + h * hd + d0);
+  }
+  for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x) vdst[(size_t)e * page_size] = vrow[e];
+}
+
 extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions, const int* token_req,
                                 const int* block_table, int table_stride, const float* inv_freq, void* k_cache,
                                 void* v_cache, int n_tokens, int heads, int kv_heads, int hd, int rot, int page_size,
@@ -217,6 +281,21 @@ extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions,
     return NS_ERR_BAD_ARG;
   const int work = heads * (rot / 2) > kv_heads * hd ? heads * (rot / 2) : kv_heads * hd;
   const int threads = work >= 1024 ? 1024 : work >= 512 ? 512 : 256;
+  const int vlen = dtype == NS_DTYPE_F32 ? 4 : 8;
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache) & 15) == 0 && row_stride % vlen == 0 && (rot / 2) % vlen == 0 &&
+                       (hd - rot) % vlen == 0 && hd % vlen == 0 && rot > 0;
+  if (aligned) {
+    const int vthreads = threads >= 512 ? 256 : threads;
+    if (dtype == NS_DTYPE_F32)
+      rope_kv_vec_kernel<float><<<n_tokens, vthreads, (size_t)(rot + 2) * sizeof(float), stream>>>((float*)qkv, row_stride, positions, token_req, block_table, table_stride,
+                                                          inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
+    else if (dtype == NS_DTYPE_BF16)
+      rope_kv_vec_kernel<bf16_t><<<n_tokens, vthreads, (size_t)(rot + 2) * sizeof(float), stream>>>((bf16_t*)qkv, row_stride, positions, token_req, block_table, table_stride,
+                                                           inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
+    else
+      return NS_ERR_UNSUPPORTED;
+    return ns_launch_status();
+  }
   if (dtype == NS_DTYPE_F32)
     rope_kv_kernel<float><<<n_tokens, threads, (size_t)(rot + 2) * sizeof(float), stream>>>((float*)qkv, row_stride, positions, token_req, block_table, table_stride,
                                                         inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
