@@ -34,17 +34,18 @@ def _require_gpu(device) -> torch.device:
     return device
 
 
-def load_model(model, device="cuda", dtype=torch.bfloat16) -> DecoderModel:
-    """``model``: a folder with config.json and safetensors files."""
+def load_model(model, device="cuda", dtype=torch.bfloat16, layouts: str = "auto") -> DecoderModel:
+    """``model``: a folder with config.json and safetensors files.  ``layouts``: see ``DecoderModel.load``."""
     folder = Path(model)
     if not folder.is_dir():
         raise FileNotFoundError(f"{model} is not a model folder (no network access is attempted)")
     config, spec = load_config(folder)
     device = _require_gpu(device)
-    return DecoderModel(spec, config).load(SafetensorsSource(folder), as_dtype(dtype), device)
+    return DecoderModel(spec, config).load(SafetensorsSource(folder), as_dtype(dtype), device, layouts)
 
 
-def random_model(config, seed: int = 0, device="cuda", dtype=torch.bfloat16, on_device: bool = False) -> DecoderModel:
+def random_model(config, seed: int = 0, device="cuda", dtype=torch.bfloat16, on_device: bool = False,
+                 layouts: str = "auto") -> DecoderModel:
     """A model with seeded random weights, without a folder.  ``on_device`` draws the numbers on the GPU
     (large models; the numbers then differ from the CPU draw of the same seed, the law does not)."""
     device = _require_gpu(device)
@@ -53,7 +54,7 @@ def random_model(config, seed: int = 0, device="cuda", dtype=torch.bfloat16, on_
     net = DecoderModel(spec, config)
     skip = {spec.head_name} if spec.tie_head else set()
     if not on_device:
-        return net.load(DictSource(random_tensors(net.wanted(), seed, dtype, skip=skip), "<random>"), dtype, device)
+        return net.load(DictSource(random_tensors(net.wanted(), seed, dtype, skip=skip), "<random>"), dtype, device, layouts)
 
     class _Lazy:
         """Draws each tensor on the device when it is asked for, so that no second copy is ever held."""
@@ -76,4 +77,4 @@ def random_model(config, seed: int = 0, device="cuda", dtype=torch.bfloat16, on_
             t = torch.empty(shape, dtype=dtype, device=device).normal_(0.0, 0.02, generator=self.gen)
             return t + 1.0 if role == "norm" else t
 
-    return net.load(_Lazy(net.wanted()), dtype, device)
+    return net.load(_Lazy(net.wanted()), dtype, device, layouts)

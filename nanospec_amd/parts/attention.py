@@ -14,7 +14,7 @@ import torch
 
 from ..kernels import ops
 from . import registry
-from .linear import LinearWeight
+from .linear import Layouts, LinearWeight
 from .needs import PagedNeed
 
 
@@ -64,7 +64,8 @@ class Attention:
         self.wqkv_rope = None
         if dtype == torch.bfloat16 and s.hidden % 8 == 0 and s.head_dim % 16 == 0 and rot % 16 == 0:
             self.wqkv_rope = ops.TiledWeight(wqkv, ops.qkv_rope_row_order(s.heads, s.kv_heads, s.head_dim, rot))
-        self.wqkv = LinearWeight(wqkv, tiled=self.wqkv_rope is None)
+        # (without the plain layout the stacked matrix is also kept tiled in its own row order, for more than 16 rows)
+        self.wqkv = LinearWeight(wqkv, tiled=self.wqkv_rope is None or not Layouts.keep_plain)
         self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous())
 
     def cache_need(self):

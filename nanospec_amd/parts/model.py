@@ -8,7 +8,7 @@ import torch
 from ..kernels import ops
 from ..weights import source as wsource
 from . import registry
-from .linear import LinearWeight
+from .linear import Layouts, LinearWeight
 from .needs import PagedNeed, StateNeed
 
 
@@ -45,14 +45,27 @@ class DecoderModel:
     def wanted(self) -> dict:
         return wanted_tensors(self.spec, self.layers)
 
-    def load(self, source, dtype: torch.dtype, device) -> "DecoderModel":
+    def load(self, source, dtype: torch.dtype, device, layouts: str = "auto") -> "DecoderModel":
         """Check the source against what the model wants (one error that lists everything wrong), then read
         each tensor once.  A head that is absent is the embedding table if the configuration ties them
-        (reference: model/loader.py:62-70)."""
+        (reference: model/loader.py:62-70).  ``layouts``: "both" keeps every bfloat16 matrix in two layouts
+        (``parts.linear.Layouts``), "tiled" only in the re-laid one, "auto" chooses by the memory that is free."""
         spec = self.spec
-        wanted = {k: v[0] for k, v in self.wanted().items()}
+        full = self.wanted()
+        wanted = {k: v[0] for k, v in full.items()}
         wsource.check(source, wanted, optional={spec.head_name} if spec.tie_head else frozenset())
         self.dtype, self.device = dtype, torch.device(device)
+        if layouts not in ("auto", "both", "tiled"):
+            raise ValueError(f"layouts={layouts!r}: use 'auto', 'both' or 'tiled'")
+        if layouts == "auto":
+            size = torch.finfo(dtype).bits // 8
+            linear = sum(size * shape[0] * shape[1] for name, (shape, role) in full.items() if role == "linear" and name != spec.head_name)
+            free = torch.cuda.mem_get_info(self.device)[0]
+            layouts = "both" if 2.2 * linear + size * 2 * spec.vocab_size * spec.hidden < 0.8 * free else "tiled"
+            if layouts == "tiled" and dtype == torch.bfloat16:
+                print(f"[nanospec_amd] {linear / 2**30:.0f} GiB of matrices, {free / 2**30:.0f} GiB free: keeping one layout; "
+                      "steps of many tokens will be slower", flush=True)
+        Layouts.keep_plain = layouts == "both"
         get = source.get
         self.embed = get(spec.embed_name).to(device=device, dtype=dtype).contiguous()
         if spec.head_name in source.names():

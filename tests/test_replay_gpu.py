@@ -168,6 +168,26 @@ def test_norms_as_kernels_of_their_own(tiny_folders, name, schedule):
         ops.linear_resid_norm = real
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_one_weight_layout_only(tiny_folders, name):
+    """Without the plain layout (models that fill the memory) steps of many tokens run in slices through the streaming
+    kernels: same logits."""
+    from nanospec_amd.loader import load_model
+    from nanospec_amd.parts.linear import Layouts
+
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, torch.bfloat16)
+    try:
+        model = load_model(folder, dtype=torch.bfloat16, layouts="tiled")
+        assert model.layers[0].ffn.down.plain is None and model.layers[0].ffn.gate_up.stacked is None
+        for make in (traces.whole, traces.tail_decoded):
+            steps, where = make(seqs)
+            replay(model, steps, where, ref, torch.bfloat16, 256, page)
+    finally:
+        Layouts.keep_plain = True
+
+
 def test_trace_run_program(tiny_folders, tmp_path):
     """bin/trace_run as a user calls it: JSON lines in, <step>.f32 out, 'done <step>' after every step."""
     name = "B"
