@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
   const int xrow0 = tid >> 4, xcol = (tid & 15) * 8;
   // A stage holds what one k tile needs from memory: this wave's fragments of w (and w2) and this thread's pieces of x.
   // DEPTH stages are in flight: the loads of k tile t + DEPTH - 1 are issued before the arithmetic of k tile t.
-  constexpr int DEPTH = NACC * NT >= 2 ? 2 : 3;
+  constexpr int DEPTH = NACC * NT >= 4 ? 2 : 3;
   struct Stage {
     bf16x8 wf[NACC][NT][4];
     bf16x8 xr[MT];
