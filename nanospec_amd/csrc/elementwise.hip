@@ -132,6 +132,85 @@ static bool launch_rmsnorm_vec(void* out, void* resid, const void* x, const void
   return true;
 }
 
+// The same where x has not been added up yet: x[r][c] = T(sum_s partial[s][r][c]), the ranges of a product whose K was
+// cut (gemm_wide.hip), added in order.  One workgroup per row; the row stays in registers between the two passes.
+// For dim a multiple of 4 and at most 4 * MAXC * threads.
+template <typename T, int MAXC>
+__global__ void rmsnorm_partial_kernel(T* __restrict__ out, T* resid, const float* __restrict__ partial, size_t plane, int ksplit,
+                                       const T* __restrict__ w, const int* __restrict__ rows, int dim, float eps, int write_resid) {
+  typedef T vec4_t __attribute__((ext_vector_type(4)));
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const size_t r = rows ? (size_t)rows[i] : (size_t)i;
+  const float4* pr = reinterpret_cast<const float4*>(partial + r * dim);
+  const size_t plane4 = plane / 4;
+  T* rr = resid ? resid + r * dim : nullptr;
+  const int n4 = dim / 4;
+  float val[MAXC][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int idx = threadIdx.x + c * blockDim.x;
+    if (idx < n4) {
+      float4 s = pr[idx];
+      for (int k = 1; k < ksplit; ++k) {
+        const float4 t = pr[(size_t)k * plane4 + idx];
+        s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+      }
+      const float xs[4] = {s.x, s.y, s.z, s.w};
+      vec4_t rv = {};
+      if (rr) rv = *reinterpret_cast<const vec4_t*>(rr + idx * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = round_to<T>(xs[e]);
+        if (rr) v = round_to<T>(to_f(rv[e]) + v);
+        val[c][e] = v;
+        ss += v * v;
+      }
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rinv = rsqrtf(ss / (float)dim + eps);
+  T* o = out + (size_t)i * dim;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int idx = threadIdx.x + c * blockDim.x;
+    if (idx < n4) {
+      const vec4_t wv = *reinterpret_cast<const vec4_t*>(w + idx * 4);
+      vec4_t rv, ov;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        rv[e] = from_f<T>(val[c][e]);
+        ov[e] = from_f<T>(to_f(wv[e]) * round_to<T>(val[c][e] * rinv));
+      }
+      if (write_resid && rr) *reinterpret_cast<vec4_t*>(rr + idx * 4) = rv;
+      *reinterpret_cast<vec4_t*>(o + idx * 4) = ov;
+    }
+  }
+}
+
+// partial: float32 [ksplit][plane / dim rows][dim].
+extern "C" int ns_rmsnorm_partial(void* out, void* resid, const void* partial, size_t plane, int ksplit, const void* w,
+                                  const int* rows, int n_rows, int dim, float eps, int write_resid, int dtype,
+                                  hipStream_t stream) {
+  if (n_rows <= 0 || dim <= 0 || (dim & 3) || ksplit < 1 || !partial || (plane & 3) || ((uintptr_t)partial & 15) ||
+      (((uintptr_t)out | (uintptr_t)resid | (uintptr_t)w) & 7))
+    return NS_ERR_BAD_ARG;
+  if (write_resid && rows) return NS_ERR_BAD_ARG;
+  if (dtype != NS_DTYPE_BF16) return NS_ERR_UNSUPPORTED;
+  const int n4 = dim / 4;
+  const int threads = n4 <= 256 ? 256 : n4 <= 2048 ? 512 : 1024;
+  const int chunks = (n4 + threads - 1) / threads;
+  if (chunks > 4) return NS_ERR_UNSUPPORTED;
+  if (chunks <= 1)
+    rmsnorm_partial_kernel<bf16_t, 1><<<n_rows, threads, 0, stream>>>((bf16_t*)out, (bf16_t*)resid, (const float*)partial, plane, ksplit, (const bf16_t*)w, rows, dim, eps, write_resid);
+  else if (chunks == 2)
+    rmsnorm_partial_kernel<bf16_t, 2><<<n_rows, threads, 0, stream>>>((bf16_t*)out, (bf16_t*)resid, (const float*)partial, plane, ksplit, (const bf16_t*)w, rows, dim, eps, write_resid);
+  else
+    rmsnorm_partial_kernel<bf16_t, 4><<<n_rows, threads, 0, stream>>>((bf16_t*)out, (bf16_t*)resid, (const float*)partial, plane, ksplit, (const bf16_t*)w, rows, dim, eps, write_resid);
+  return ns_launch_status();
+}
+
 extern "C" int ns_rmsnorm(void* out, void* resid, const void* x, const void* w, const int* rows, int n_rows, int dim,
                           float eps, int write_resid, int dtype, hipStream_t stream) {
   if (n_rows <= 0 || dim <= 0 || (!resid && !x)) return NS_ERR_BAD_ARG;

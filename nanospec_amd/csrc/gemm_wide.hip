@@ -190,8 +190,11 @@ static int launch_wide(float* partial, const bf16_t* x, const bf16_t* wt, const 
 }
 
 // workspace: (wt2 ? 2 : 1) * ksplit * M * N floats (unused with ksplit == 1).  epi 0: store; 1: silu(x.w^T) * (x.w2^T).
+// defer (with ksplit > 1 and epi 0): the ranges stay in the workspace as [ksplit][M][N] and nothing is written to out; they
+// are added later by ns_wide_reduce or by a norm that reads them (ns_rmsnorm_partial).
 extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
-                                 int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, hipStream_t stream) {
+                                 int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer,
+                                 hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
   if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
   const int KT = (K + 127) / 128;
@@ -207,6 +210,7 @@ extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, cons
     default: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
   }
   if (st != NS_OK || direct) return st;
+  if (defer) return epi == 0 ? NS_OK : NS_ERR_BAD_ARG;
   const size_t total = (size_t)M * N;
   const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
   if (epi == 1)
@@ -215,5 +219,18 @@ extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, cons
     gemm_wide_reduce_kernel<float, 0><<<blocks, 256, 0, stream>>>((float*)out, part, M, N, out_stride, ksplit);
   else
     gemm_wide_reduce_kernel<bf16_t, 0><<<blocks, 256, 0, stream>>>((bf16_t*)out, part, M, N, out_stride, ksplit);
+  return ns_launch_status();
+}
+
+// out[m][n] = sum over the ranges of partial[s][m][n], added in order.
+extern "C" int ns_wide_reduce(void* out, const void* partial, int M, int N, int out_stride, int ksplit, int out_f32,
+                              hipStream_t stream) {
+  if (M <= 0 || N <= 0 || ksplit < 1 || out_stride < N || !out || !partial) return NS_ERR_BAD_ARG;
+  const size_t total = (size_t)M * N;
+  const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+  if (out_f32)
+    gemm_wide_reduce_kernel<float, 0><<<blocks, 256, 0, stream>>>((float*)out, (const float*)partial, M, N, out_stride, ksplit);
+  else
+    gemm_wide_reduce_kernel<bf16_t, 0><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const float*)partial, M, N, out_stride, ksplit);
   return ns_launch_status();
 }

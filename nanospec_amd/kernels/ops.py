@@ -73,10 +73,50 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = Non
     return out
 
 
-def rmsnorm(weight: torch.Tensor, eps: float, resid: torch.Tensor | None = None, x: torch.Tensor | None = None,
+class PartialSums:
+    """A product whose K was cut into ranges that have not been added up yet (``linear_wide(..., defer=True)``):
+    ``ws`` holds float32 [ksplit, rows, n].  ``rmsnorm`` adds them while it reads them; ``reduce_partial`` makes the tensor."""
+
+    def __init__(self, ws: torch.Tensor, ksplit: int, rows: int, n: int, dtype: torch.dtype) -> None:
+        self.ws, self.ksplit, self.rows, self.n, self.dtype = ws, ksplit, rows, n, dtype
+        self.shape = (rows, n)
+
+
+def reduce_partial(p: PartialSums, out: torch.Tensor | None = None) -> torch.Tensor:
+    """The sum of the ranges, in order, rounded to the product's dtype."""
+    _gpu(p.ws, out)
+    if out is None:
+        out = torch.empty((p.rows, p.n), dtype=p.dtype, device=p.ws.device)
+    if out.shape != (p.rows, p.n) or out.stride(1) != 1 or out.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelRefused("reduce_partial: out has the wrong shape or dtype")
+    _check(build.core().ns_wide_reduce(_ptr(out), _ptr(p.ws), c_int(p.rows), c_int(p.n), c_int(out.stride(0)), c_int(p.ksplit),
+                                       c_int(1 if out.dtype == torch.float32 else 0), _stream()), "reduce_partial")
+    return out
+
+
+def rmsnorm(weight: torch.Tensor, eps: float, resid: torch.Tensor | None = None, x: "torch.Tensor | PartialSums | None" = None,
             rows: torch.Tensor | None = None, write_resid: bool = False, out: torch.Tensor | None = None) -> torch.Tensor:
     """out[i] = weight * norm(resid[r] + x[r]) with r = rows[i] (or i).  With ``write_resid`` the sum
-    is also stored back into ``resid`` (not with ``rows``)."""
+    is also stored back into ``resid`` (not with ``rows``).  ``x`` may be a ``PartialSums``."""
+    if isinstance(x, PartialSums):
+        p, dim = x, weight.numel()
+        ok = (weight.dtype == torch.bfloat16 and p.dtype == torch.bfloat16 and p.n == dim and dim % 4 == 0 and dim <= 16384
+              and (resid is None or (resid.shape == (p.rows, dim) and resid.is_contiguous() and resid.dtype == weight.dtype)))
+        if not ok:
+            x = reduce_partial(p)
+        else:
+            _gpu(weight, resid, rows, p.ws)
+            if rows is not None:
+                _i32(rows, "rows")
+            n = rows.numel() if rows is not None else p.rows
+            if out is None:
+                out = torch.empty((n, dim), dtype=weight.dtype, device=weight.device)
+            if out.shape != (n, dim) or not out.is_contiguous() or out.dtype != weight.dtype:
+                raise KernelRefused("rmsnorm: out has the wrong shape")
+            _check(build.core().ns_rmsnorm_partial(_ptr(out), _ptr(resid), _ptr(p.ws), c_size_t(p.rows * dim), c_int(p.ksplit), _ptr(weight),
+                                                   _ptr(rows), c_int(n), c_int(dim), c_float(eps), c_int(1 if write_resid else 0),
+                                                   c_int(_dtype_code(weight)), _stream()), "rmsnorm")
+            return out
     src = resid if resid is not None else x
     if src is None:
         raise KernelRefused("rmsnorm needs resid or x")
@@ -310,34 +350,37 @@ def wide_plan(n: int, k: int) -> tuple[int, int]:
 
 
 def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
-                out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0) -> torch.Tensor:
+                out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0, defer: bool = False):
     """bfloat16 x @ w.T for up to 64 rows from a tiled weight, with the tile of x shared through LDS by the four waves of
     a workgroup and K cut into ``ksplit`` ranges that a second kernel adds up; with ``w2``: silu(x @ w.T) * (x @ w2.T).
-    ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values (none for a single range)."""
+    ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values (none for a single range).  ``defer`` (not with
+    ``w2``): with more than one range the second kernel is left out and a ``PartialSums`` over the workspace comes back."""
     _gpu(x, out, workspace)
     if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k):
         raise KernelRefused(f"linear_wide takes bfloat16 x [rows <= {SKINNY_MAX_ROWS}, {w.k}] with an inner size that is a "
                             f"multiple of 8; got {tuple(x.shape)} {x.dtype}")
     m = x.shape[0]
     want = torch.float32 if out_f32 else x.dtype
-    if out is None:
+    plan = wide_plan(w.n, w.k)
+    ksplit, nt = ksplit or plan[0], nt or plan[1]
+    defer = defer and ksplit > 1 and w2 is None and not out_f32
+    if out is None and not defer:
         out = torch.empty((m, w.n), dtype=want, device=x.device)
-    if out.shape != (m, w.n) or out.dtype != want or out.stride(1) != 1:
+    if not defer and (out.shape != (m, w.n) or out.dtype != want or out.stride(1) != 1):
         raise KernelRefused("linear_wide: out has the wrong shape or dtype")
     if w2 is not None and (w2.n != w.n or w2.k != w.k or out_f32):
         raise KernelRefused("linear_wide: w2 must match w and the gated result is bfloat16")
-    plan = wide_plan(w.n, w.k)
-    ksplit, nt = ksplit or plan[0], nt or plan[1]
     need = (2 if w2 is not None else 1) * ksplit * m * w.n if ksplit > 1 else 0  # a single range writes the result itself
     if workspace is None and need:
         workspace = torch.empty(need, dtype=torch.float32, device=x.device)
     if need and (workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous()):
         raise KernelRefused("linear_wide: workspace too small")
-    _check(build.core().ns_gemm_wide_bf16(_ptr(out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None),
-                                          c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
-                                          c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), _stream()),
+    _check(build.core().ns_gemm_wide_bf16(_ptr(None if defer else out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data),
+                                          _ptr(w2.data if w2 is not None else None), c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)),
+                                          c_int(w.n if defer else out.stride(0)), c_int(1 if w2 is not None else 0),
+                                          c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), c_int(1 if defer else 0), _stream()),
            "linear_wide")
-    return out
+    return PartialSums(workspace, ksplit, m, w.n, x.dtype) if defer else out
 
 
 def qkv_rope_row_order(heads: int, kv_heads: int, head_dim: int, rotary_dim: int) -> torch.Tensor:

@@ -20,6 +20,7 @@ from .needs import PagedNeed
 
 class Attention:
     graph_safe = True
+    ends_in_residual = True  # forward takes residual=IntoResidual
 
     def __init__(self, spec, prefix: str) -> None:
         if spec.heads % spec.kv_heads:

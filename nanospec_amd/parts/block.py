@@ -43,41 +43,45 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
-    links_blocks = True  # forward takes next_norm and next_sums
+    links_blocks = True  # forward takes next_norm, next_sums and next_carry
 
-    def forward(self, ctx, resid, delta, cache, owns_cache, delta_out, next_norm=None, next_sums=None):
-        """``delta``: what the block before left to be added (a tensor, or None at the start), or a ``PreNormed``: then
-        ``resid`` is already whole and the first norm's input comes ready for a product that ``links_norms``.
-        ``next_norm``: the norm that will read this block's result (the next block's first one), if it
-        ``links_products``; ``next_sums``: float32 [tokens, ceil(width / 16)] that lives as long as the step.
-        -> None, with the block's not yet added output in ``delta_out``; or a ``PreNormed`` for ``next_norm`` (its rows
-        in ``delta_out``, its sums in ``next_sums``), with ``resid`` whole."""
+    def forward(self, ctx, resid, delta, cache, owns_cache, delta_out, next_norm=None, next_sums=None, next_carry=None):
+        """``delta``: what the block before left to be added: a tensor (None at the start), a ``PartialSums``, or a
+        ``PreNormed``, in which case ``resid`` is already whole and the first norm's input comes ready for a product that
+        ``links_norms``.  ``next_norm``: the norm that will read this block's result (the next block's first one), if it
+        ``links_products``; ``next_sums`` (float32 [tokens, ceil(width / 16)]) and ``next_carry`` (float32, 16 * tokens *
+        width, or None): buffers that live as long as the step.
+        -> None, with the block's not yet added output in ``delta_out``; or that output in one of the forms of
+        ``IntoResidual`` (a tensor is then ``delta_out``)."""
         n = resid.shape[0]
         mark = ctx.arena.mark()
         link = getattr(ctx, "link_norms", False) and resid.dtype == torch.bfloat16
-        can = lambda part: link and getattr(part, "links_norms", lambda rows: False)(n)
+        takes = lambda part: link and getattr(part, "links_norms", lambda rows: False)(n)  # a PreNormed input
+        ends = lambda part: link and getattr(part, "ends_in_residual", False)
         lp = lambda norm: link and norm is not None and getattr(norm, "links_products", False) and norm.weight.dtype == resid.dtype
+        buf = lambda: ctx.arena.take(resid.shape, resid.dtype)
 
         # first norm and mixer
         if isinstance(delta, ops.PreNormed):
-            h = delta if can(self.mixer) else self.mixer_norm.forward(ctx, resid=resid, out=ctx.arena.take(resid.shape, resid.dtype))
+            h = delta if takes(self.mixer) else self.mixer_norm.forward(ctx, resid=resid, out=buf())
         else:
-            h = self.mixer_norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None,
-                                        out=ctx.arena.take(resid.shape, resid.dtype))
-        if can(self.mixer) and lp(self.ffn_norm):
-            h2 = self.mixer.forward(ctx, h, cache, owns_cache, residual=IntoResidual(resid, self.ffn_norm.weight, self.ffn_norm.spec.eps))
-            if not can(self.ffn):
-                h2 = self.ffn_norm.forward(ctx, resid=resid, out=ctx.arena.take(resid.shape, resid.dtype))
+            h = self.mixer_norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None, out=buf())
+        if ends(self.mixer) and lp(self.ffn_norm):
+            a = self.mixer.forward(ctx, h, cache, owns_cache, residual=IntoResidual(resid, self.ffn_norm.weight, self.ffn_norm.spec.eps))
         else:
-            a = self.mixer.forward(ctx, h, cache, owns_cache, out=ctx.arena.take(resid.shape, resid.dtype))
-            h2 = self.ffn_norm.forward(ctx, resid=resid, x=a, write_resid=True, out=ctx.arena.take(resid.shape, resid.dtype))
+            a = self.mixer.forward(ctx, h, cache, owns_cache, out=buf())
 
         # second norm and feed-forward
-        if can(self.ffn) and lp(next_norm) and next_sums is not None:
-            # what the next block reads must outlive this block's scratch: it goes into delta_out and next_sums
-            pre = self.ffn.forward(ctx, h2, residual=IntoResidual(resid, next_norm.weight, next_norm.spec.eps, delta_out, next_sums))
+        if isinstance(a, ops.PreNormed):
+            h2 = a if takes(self.ffn) else self.ffn_norm.forward(ctx, resid=resid, out=buf())
+        else:
+            h2 = self.ffn_norm.forward(ctx, resid=resid, x=a, write_resid=True, out=buf())
+        if ends(self.ffn) and lp(next_norm) and next_sums is not None:
+            # what the next block reads must outlive this block's scratch
+            out = self.ffn.forward(ctx, h2, residual=IntoResidual(resid, next_norm.weight, next_norm.spec.eps, delta_out, next_sums,
+                                                                 next_carry, outlives=True))
             ctx.arena.release(mark)
-            return pre
+            return out
         self.ffn.forward(ctx, h2, out=delta_out)
         ctx.arena.release(mark)
         return None

@@ -33,15 +33,21 @@ WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the libr
 
 
 class IntoResidual:
-    """Asks a part to end in ``resid += output`` (in place) and to hand back what the RMS norm after it needs
-    (``kernels.ops.PreNormed``), instead of returning its output: the part's last product then does the work of the
-    residual sum and of the norm's statistics.  ``next_weight``, ``eps``: that norm's weight and epsilon.  ``x_next``
-    (like resid) and ``ssq`` (float32 [rows, ceil(width / 16)]): where to put them, if they must outlive the step's
-    scratch."""
+    """Asks a part to hand its output to the residual stream and the RMS norm after it in the cheapest form its last
+    product has, instead of returning a finished tensor:
+      * ``kernels.ops.PreNormed``: ``resid += output`` has been done in place and the norm needs no kernel of its own
+        (at most 16 rows: the product's epilogue did the sum and the norm's statistics);
+      * ``kernels.ops.PartialSums``: the ranges of a product whose K was cut, which the norm kernel adds up as it reads
+        them (17 to 64 rows);
+      * a tensor: the output, still to be added by the norm kernel.
+    ``next_weight``, ``eps``: that norm's weight and epsilon.  ``x_next`` (like resid), ``ssq`` (float32 [rows,
+    ceil(width / 16)]) and ``carry`` (float32, 16 * rows * width): where the results go if they must outlive the block's
+    scratch (``outlives``); otherwise scratch is taken."""
 
     def __init__(self, resid: torch.Tensor, next_weight: torch.Tensor, eps: float, x_next: torch.Tensor | None = None,
-                 ssq: torch.Tensor | None = None) -> None:
-        self.resid, self.next_weight, self.eps, self.x_next, self.ssq = resid, next_weight, eps, x_next, ssq
+                 ssq: torch.Tensor | None = None, carry: torch.Tensor | None = None, outlives: bool = False) -> None:
+        self.resid, self.next_weight, self.eps = resid, next_weight, eps
+        self.x_next, self.ssq, self.carry, self.outlives = x_next, ssq, carry, outlives
 
 
 class LinearWeight:
@@ -60,17 +66,27 @@ class LinearWeight:
         """Whether a product of ``rows`` rows can take a ``PreNormed`` input and can end in the residual stream."""
         return self.tiled is not None and rows <= STREAM_ROWS
 
-    def into_residual(self, x: torch.Tensor, link: IntoResidual, arena=None) -> "ops.PreNormed":
-        """link.resid += x @ W^T; -> what the norm after it needs."""
-        if not self.links_norms(x.shape[0]):
-            raise ops.KernelRefused("this product cannot end in the residual stream (rows, layout or precision)")
+    def into_residual(self, x: torch.Tensor, link: IntoResidual, arena=None):
+        """x @ W^T on its way into the residual stream, in one of the three forms ``IntoResidual`` names."""
         m = x.shape[0]
-        x_next, ssq = link.x_next, link.ssq
-        if x_next is None and arena is not None:
-            x_next = arena.take(tuple(link.resid.shape), link.resid.dtype)
-        if ssq is None and arena is not None:
-            ssq = arena.take((m, -(-self.n // 16)), torch.float32)
-        return ops.linear_resid_norm(x, self.tiled, link.resid, link.next_weight, link.eps, x_next=x_next, ssq=ssq)
+        take = (lambda shape, dtype: arena.take(shape, dtype)) if arena is not None else (lambda shape, dtype: torch.empty(shape, dtype=dtype, device=x.device))
+        if self.links_norms(m) and x.dtype == torch.bfloat16 and ops.tiled_takes(x[:1], self.k):
+            x_next = link.x_next if link.x_next is not None else take(tuple(link.resid.shape), link.resid.dtype)
+            ssq = link.ssq if link.ssq is not None else take((m, -(-self.n // 16)), torch.float32)
+            return ops.linear_resid_norm(x, self.tiled, link.resid, link.next_weight, link.eps, x_next=x_next, ssq=ssq)
+        if (self.tiled is not None and STREAM_ROWS < m <= ops.SKINNY_MAX_ROWS and (self.plain is None or self.n <= WIDE_MAX_N)
+                and x.dtype == torch.bfloat16 and ops.tiled_takes(x[:1], self.k)):
+            ksplit, nt = ops.wide_plan(self.n, self.k)
+            need = ksplit * m * self.n
+            ws = None
+            if ksplit > 1 and link.carry is not None and link.carry.numel() >= need:
+                ws = link.carry
+            elif ksplit > 1 and not link.outlives:
+                ws = take((need,), torch.float32)
+            if ws is not None:
+                return ops.linear_wide(x, self.tiled, workspace=ws, ksplit=ksplit, nt=nt, defer=True)
+        out = link.x_next if link.x_next is not None else take((m, self.n), x.dtype)
+        return self(x, out=out, arena=arena)
 
     def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None) -> torch.Tensor:
         """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated.

@@ -89,16 +89,21 @@ class DecoderModel:
         ops.embed(self.embed, ctx.token_ids, out=resid)
         pending = None
         order = self.spec.run_order
-        sums = ctx.arena.take((n, -(-self.spec.hidden // 16)), torch.float32)  # see PreNormBlock.forward
+        # buffers for what one block hands to the next (see PreNormBlock.forward)
+        sums = ctx.arena.take((n, -(-self.spec.hidden // 16)), torch.float32)
+        carry = ctx.arena.take((16 * n * self.spec.hidden,), torch.float32) if 16 < n <= ops.SKINNY_MAX_ROWS and self.dtype == torch.bfloat16 else None
         for i, call in enumerate(order):
             layer = self.layers[call.layer]
             if getattr(layer, "links_blocks", False) and i + 1 < len(order):
                 # the norm that reads this block's result is the next block's first
                 nxt = getattr(self.layers[order[i + 1].layer], "mixer_norm", None)
-                out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta, next_norm=nxt, next_sums=sums)
+                out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta, next_norm=nxt, next_sums=sums,
+                                    next_carry=carry)
             else:
                 if isinstance(pending, ops.PreNormed):
                     pending = None  # resid is whole already; a block that does not know the hand-over starts from it
+                elif isinstance(pending, ops.PartialSums):
+                    pending = ops.reduce_partial(pending, out=delta)
                 out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta)
             pending = out if out is not None else delta
         return resid, pending

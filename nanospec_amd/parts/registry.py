@@ -24,9 +24,10 @@ What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are 
 
 Optional, for parts whose products can do the work of the RMS norms around them (``parts.linear.IntoResidual``):
   norm         links_products = True, weight, spec.eps
-  mixer, ffn   links_norms(rows) -> bool; forward(..., residual=IntoResidual) -> kernels.ops.PreNormed, and x may be
-               a PreNormed
-  block        links_blocks = True; forward(..., next_norm=None, next_sums=None) -> None | PreNormed
+  mixer, ffn   ends_in_residual = True: forward(..., residual=IntoResidual) -> PreNormed | PartialSums | tensor;
+               links_norms(rows) -> bool: x may be a PreNormed
+  block        links_blocks = True; forward(..., next_norm=None, next_sums=None, next_carry=None) -> None or one of
+               those three
 """
 
 from __future__ import annotations

@@ -11,6 +11,7 @@ from .linear import GatedWeights, LinearWeight
 
 class SwiGLU:
     graph_safe = True
+    ends_in_residual = True  # forward takes residual=IntoResidual
 
     def __init__(self, spec, prefix: str) -> None:
         self.spec, self.prefix = spec, prefix

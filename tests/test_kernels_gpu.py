@@ -276,6 +276,39 @@ def test_product_that_updates_the_residual_and_feeds_the_next_norm(m, hidden, in
     assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * up).max() <= 2.0
 
 
+@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("hidden,inner,ksplit", [(136, 1024, 4), (4096, 1024, 2), (72, 512, 3)])
+def test_ranges_of_a_product_added_by_the_norm_that_reads_them(m, hidden, inner, ksplit):
+    """The 17-to-64-row product leaves the ranges of K unadded; the RMS norm adds them as it reads them, with the residual
+    sum and with a row gather; ``reduce_partial`` gives the same tensor as the product run whole."""
+    ops = _ops()
+    torch.manual_seed(m + hidden)
+    eps = 1e-5
+    x = torch.randn(m, inner).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(hidden, inner) / math.sqrt(inner)).to(torch.bfloat16).to(DEV)
+    wt = ops.TiledWeight(w)
+    resid0 = torch.randn(m, hidden).to(torch.bfloat16)
+    w_norm = (1 + 0.2 * torch.randn(hidden)).to(torch.bfloat16)
+    part = ops.linear_wide(x, wt, ksplit=ksplit, nt=1, defer=True)
+    assert isinstance(part, ops.PartialSums) and part.ws.numel() >= ksplit * m * hidden
+    whole = ops.linear_wide(x, wt, ksplit=ksplit, nt=1)
+    assert torch.equal(ops.reduce_partial(part), whole)
+    # sum + norm
+    resid = resid0.to(DEV).clone()
+    out = ops.rmsnorm(w_norm.to(DEV), eps, resid=resid, x=part, write_resid=True)
+    resid_ref = resid0.to(DEV).clone()
+    ref = ops.rmsnorm(w_norm.to(DEV), eps, resid=resid_ref, x=whole, write_resid=True)
+    assert torch.equal(resid, resid_ref)
+    assert ulps_of_row_max(out.cpu(), ref.cpu().float()).max() <= 1.0
+    want = pl.rms_norm((resid0.float() + whole.cpu().float()).to(torch.bfloat16), w_norm, eps)
+    assert ulps_of_row_max(out.cpu(), want.float()).max() <= 1.0
+    # gathered rows, no residual
+    rows = torch.tensor([m - 1, 0, 5], dtype=torch.int32, device=DEV)
+    got = ops.rmsnorm(w_norm.to(DEV), eps, x=part, rows=rows)
+    want = pl.rms_norm(whole.cpu()[rows.cpu().long()], w_norm, eps)
+    assert ulps_of_row_max(got.cpu(), want.float()).max() <= 1.0
+
+
 def test_qkv_product_takes_a_prenormed_input():
     ops = _ops()
     torch.manual_seed(3)

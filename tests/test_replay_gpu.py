@@ -231,7 +231,7 @@ def llama_1b_slice(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-def test_real_shape_slice_matches_plain(llama_1b_slice, dtype):
+def test_real_shape_slice_matches_plain(llama_1b_slice, dtype, request):
     """The kernels at the sizes of a real model (head size 64, a vocabulary of 128256, width 2048): one request whole with
     its last tokens decoded, one in portions, mixed in one batch, at positions where the llama3 scaling matters."""
     from nanospec_amd.engine.replay import Replayer
@@ -243,6 +243,22 @@ def test_real_shape_slice_matches_plain(llama_1b_slice, dtype):
     ref = {r: pl.logits_of_sequence(w, cfg, t, dtype) for r, t in seqs.items()}
     model = load_model(folder, dtype=dtype)
     rep = Replayer(model, 384, page_size=16)
+    from nanospec_amd.kernels import ops
+
+    seen = {"unadded": 0, "linked": 0}
+    real_wide, real_link = ops.linear_wide, ops.linear_resid_norm
+
+    def wide(*a, **k):
+        out = real_wide(*a, **k)
+        seen["unadded"] += isinstance(out, ops.PartialSums)
+        return out
+
+    def linked(*a, **k):
+        seen["linked"] += 1
+        return real_link(*a, **k)
+
+    ops.linear_wide, ops.linear_resid_norm = wide, linked
+    request.addfinalizer(lambda: (setattr(ops, "linear_wide", real_wide), setattr(ops, "linear_resid_norm", real_link)))
 
     def step(entries, end=()):
         out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(wants)} for r, s, e, wants in entries], list(end))
@@ -257,3 +273,8 @@ def test_real_shape_slice_matches_plain(llama_1b_slice, dtype):
         step([("a", p, p + 1, [0]), ("b", q, q + 2, [0, 1])], end=["a"] if p == 149 else [])
     step([("b", 75, 83, list(range(8)))], end=["b"])
     rep.manager.check()
+    if dtype == torch.bfloat16:
+        # the step of 38 tokens handed unadded ranges to the norms, the steps of up to 16 tokens linked norms and products
+        assert seen["unadded"] > 0 and seen["linked"] > 0, seen
+    else:
+        assert seen == {"unadded": 0, "linked": 0}
