@@ -153,7 +153,15 @@ __global__ void rmsnorm_partial_kernel(T* __restrict__ out, T* resid, const floa
     const int idx = threadIdx.x + c * blockDim.x;
     if (idx < n4) {
       float4 s = pr[idx];
-      for (int k = 1; k < ksplit; ++k) {
+      int k = 1;
+      for (; k + 3 < ksplit; k += 4) {  // four ranges' loads in flight, added in order
+        float4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = pr[(size_t)(k + u) * plane4 + idx];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { s.x += t[u].x; s.y += t[u].y; s.z += t[u].z; s.w += t[u].w; }
+      }
+      for (; k < ksplit; ++k) {
         const float4 t = pr[(size_t)k * plane4 + idx];
         s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
       }
