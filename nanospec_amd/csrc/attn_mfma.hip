@@ -402,6 +402,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 // of up to four query heads of one key/value head, one head per wave.  The four waves need the same keys and values,
 // so each block of 32 keys is fetched once per workgroup, a quarter by each wave, and handed round through LDS;
 // the next block is on its way from memory (and its page ids one block further ahead) while this one is used.
+// A tile's keys are walked by two such sets of four waves at once, each taking half of the blocks; their results are
+// joined in LDS at the end.  The longest tiles set the time of a causal prompt, and this halves their chain of blocks.
 //   keys in LDS:   row 16 t + 4 a + b holds key 8 a + 4 t + b of the block, so that the scores a lane gets from the
 //                  two 16-key products are those of keys 8 g .. 8 g + 7: the order in which it then needs the values
 //   values in LDS: [channel][32 keys], as the pages hold them
@@ -416,21 +418,22 @@ constexpr int CPR = PS / 8 < 4 ? PS / 8 : 4;  // 16-byte pieces of a block that 
 
 // Two waves per SIMD: with more registers the compiler parks the sums in accumulation registers and moves them to and
 // fro around every rescaling.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnParams a) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnParams a) {
   if constexpr (SHARED_OK) {
-    __shared__ __align__(16) bf16_t lk[2][32 * KROW];
-    __shared__ __align__(16) bf16_t lv[2][HD * VROW];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int K_BYTES = 32 * KROW * 2, V_BYTES = HD * VROW * 2, SET_BYTES = 2 * (K_BYTES + V_BYTES);
+    constexpr int JOIN_BYTES = 256 * (2 * DT * 4 + 4) * 4;  // what the second set hands to the first: sums, maxima, totals
+    __shared__ __align__(16) char smem[2 * SET_BYTES > JOIN_BYTES ? 2 * SET_BYTES : JOIN_BYTES];
+    const int half = threadIdx.x >> 8;  // which set of four waves, i.e. which half of the tile's blocks
+    bf16_t(*lk)[32 * KROW] = reinterpret_cast<bf16_t(*)[32 * KROW]>(smem + half * SET_BYTES);
+    bf16_t(*lv)[HD * VROW] = reinterpret_cast<bf16_t(*)[HD * VROW]>(smem + half * SET_BYTES + 2 * K_BYTES);
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int G = a.heads / a.kv_heads;
     const int hblks = (G + 3) / 4;
     const int ny = a.kv_heads * hblks;
     const int y = blockIdx.x % ny;
-    // Tiles are listed in the order of the tokens and the last ones see the most keys.  The first half of the workgroups
-    // takes the later half of the tiles, longest first, the second half the earlier tiles, shortest first: two
-    // workgroups that are half a grid apart, which tend to share a compute unit, then have a constant amount of work.
-    const int w = blockIdx.x / ny, longs = (a.n_tiles + 1) / 2;
-    const int tile = w < longs ? a.n_tiles - 1 - w : w - longs;
+    // tiles are listed in the order of the tokens; the last ones see the most keys, so they start first
+    const int tile = a.n_tiles - 1 - blockIdx.x / ny;
     const int kvh = y / hblks, hin = (y % hblks) * 4 + wave;
     const bool head_ok = hin < G;  // a wave without a head still fetches its share of the keys and values
     const int head = kvh * G + (head_ok ? hin : 0);
@@ -455,7 +458,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int wlo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
     const int full_hi = first_pos;                                                  // keys <= full_hi are seen by every token
     const int full_lo = a.window > 0 ? max(0, last_pos - a.window + 1) : 0;         // ... if they are >= full_lo
-    const int kb0 = wlo / 32, kb1 = (whi + 31) / 32;
+    const int tile_kb0 = wlo / 32, tile_kb1 = (whi + 31) / 32;
+    const int steps = (tile_kb1 - tile_kb0 + 1) / 2;  // blocks of the first set; the second has as many or one fewer
+    const int kb0 = half ? tile_kb0 + steps : tile_kb0, kb1 = half ? tile_kb1 : tile_kb0 + steps;
 
     bf16x8 qw[2][NQ];
 #pragma unroll
@@ -637,16 +642,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       put(0);
     }
     __syncthreads();
-    for (int kb = kb0; kb < kb1; ++kb) {
-      const int buf = (kb - kb0) & 1;
+    for (int it = 0; it < steps; ++it) {  // both sets pass every barrier; the second may have no block in the last round
+      const int kb = kb0 + it;
+      const int buf = it & 1;
       const bool more = kb + 1 < kb1;
       if (more) {
         fetch(kb + 1);
         if (kb + 2 < kb1) fetch_pages(kb + 2);
       }
-      if (head_ok) block(buf, kb);
+      if (head_ok && kb < kb1) block(buf, kb);
       if (more) put(buf ^ 1);
       __syncthreads();
+    }
+
+    // The second set hands its sums to the first, lane by lane (both hold the same columns and channels):
+    // o = o_0 2^((m_0 - m*) scale) + o_1 2^((m_1 - m*) scale), likewise the totals, m* = max(m_0, m_1).
+    float* join = reinterpret_cast<float*>(smem) + tid * (2 * DT * 4 + 4);
+    if (half) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(join + (u * DT + dt) * 4) = o[u][dt];
+        join[2 * DT * 4 + u] = m[u];
+        join[2 * DT * 4 + 2 + u] = lsum[u];
+      }
+    }
+    __syncthreads();
+    if (half) return;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const float m1 = join[2 * DT * 4 + u], l1 = join[2 * DT * 4 + 2 + u];
+      const float mstar = fmaxf(m[u], m1);
+      const float msafe = mstar == -INFINITY ? 0.f : mstar;
+      const float w0 = fast_exp2((m[u] - msafe) * a.scale_log2), w1 = fast_exp2((m1 - msafe) * a.scale_log2);
+      lsum[u] = lsum[u] * w0 + l1 * w1;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(join + (u * DT + dt) * 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[u][dt][j] = o[u][dt][j] * w0 + v[j] * w1;
+      }
     }
 
 #pragma unroll
@@ -750,7 +785,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (qt == 2 && SHARED_OK) {
     const long wgs = (long)n_tiles * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
-    attn_prefill_kernel<<<(unsigned)wgs, 256, 0, stream>>>(a);
+    attn_prefill_kernel<<<(unsigned)wgs, 512, 0, stream>>>(a);
   } else if (qt == 2)
     attn_mfma_kernel<2, false, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
   else if (coop)
