@@ -390,6 +390,8 @@ CASES = {
     "long": ([300, 0, 511], [1, 70, 1]),
     # more than 64 pages a request at every page size: the kernels hold 64 page ids at a time
     "beyond64pages": ([1300, 0], [1, 1100]),
+    # a decode row and a late portion of a prompt nine thousand tokens in: many reloads of the page ids, long key ranges
+    "far": ([9000, 8990], [1, 70]),
 }
 
 
