@@ -3,6 +3,8 @@ the output head (reference: model/llama.py:211-286).  Nothing here knows an arch
 
 from __future__ import annotations
 
+import sys
+
 import torch
 
 from ..kernels import ops
@@ -64,7 +66,7 @@ class DecoderModel:
             layouts = "both" if 2.2 * linear + size * 2 * spec.vocab_size * spec.hidden < 0.8 * free else "tiled"
             if layouts == "tiled" and dtype == torch.bfloat16:
                 print(f"[nanospec_amd] {linear / 2**30:.0f} GiB of matrices, {free / 2**30:.0f} GiB free: keeping one layout; "
-                      "steps of many tokens will be slower", flush=True)
+                      "steps of many tokens will be slower", file=sys.stderr, flush=True)
         Layouts.keep_plain = layouts == "both"
         get = source.get
         self.embed = get(spec.embed_name).to(device=device, dtype=dtype).contiguous()
