@@ -160,6 +160,41 @@ def test_preemption_gives_the_same_tokens(tiny_folders):
     assert [r.out_tokens for r in rough] == [r.out_tokens for r in calm]
 
 
+@pytest.mark.parametrize("policy,graphs,lookahead", [("preempt", True, True), ("reserve", True, True), ("preempt", False, False)])
+def test_requests_arriving_over_time_in_a_pool_that_is_too_small(tiny_folders, policy, graphs, lookahead):
+    """Thirty requests of random lengths arrive a few per step into a pool that holds a handful of them: whatever is
+    preempted, recomputed, looked ahead or replayed from a graph, every request's tokens are the plain implementation's,
+    and no page is lost."""
+    import random
+
+    from nanospec_amd import Engine, EngineConfig, SamplingParams
+
+    rnd = random.Random(4)
+    folder = tiny_folders["A"]
+    cfg, w = pl.read_config(folder), pl.read_weights(folder, torch.float32)
+    eng = Engine(model_of(folder, "A", torch.float32),
+                 EngineConfig(num_blocks=40, block_size=4, max_admit=5, max_running=12, max_step_tokens=48, prefill_chunk=20,
+                              on_exhaustion=policy, cuda_graphs=graphs, lookahead=lookahead))
+    todo = [(random_tokens(rnd.randint(1, 50), 256, 1000 + i), rnd.randint(1, 20)) for i in range(30)]
+    arriving, live, steps = iter(todo), [], 0
+    while len(live) < len(todo) or eng.has_work:
+        for _ in range(rnd.randint(0, 2)):
+            nxt = next(arriving, None)
+            if nxt is not None:
+                live.append(eng.add(nxt[0], SamplingParams(max_tokens=nxt[1])))
+        if eng.has_work:
+            eng.step()
+            steps += 1
+            if steps % 20 == 0:
+                eng.cache.check()
+    eng.cache.check()
+    assert eng.cache.num_free(0) == 40 - (1 if graphs else 0)  # all but the page of the captured graphs' pad rows
+    if policy == "preempt":
+        assert sum(r.preemptions for r in live) > 0
+    for r, (prompt, n_new) in zip(live, todo):
+        assert r.out_tokens == pl.greedy_continuation(w, cfg, prompt, n_new, torch.float32)[0], (prompt, r.preemptions)
+
+
 def test_temperature_sampling_is_seeded_and_batch_independent(tiny_folders):
     """Per-request generators (reference sched/scheduler.py:64): the same seed gives the same tokens alone or in a batch;
     the first token is the inverse-CDF draw of the plain implementation for the request's first uniform number."""
