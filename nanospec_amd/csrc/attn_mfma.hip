@@ -43,7 +43,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 // A tile descriptor, filled on the host: {request, first token of the tile among the request's tokens of this step
 // (tiles of one request follow each other every 16 qt / hp tokens),
-// row of the request's first token in the batch, tokens of the request in this step, keys after this step, 0, 0, 0}.
+// row of the request's first token in the batch, tokens of the request in this step, keys after this step,
+// for decode tiles the keys that all decode rows of the step read together, 0, 0}.
 struct AttnParams {
   bf16_t* out;        // [tokens, heads, HD]
   float* part_o;      // [n_tiles * (16 / hp) * heads, splits, HD]   (splits > 1)
@@ -71,6 +72,12 @@ __device__ __forceinline__ int wave_min_i(int v) {
   return v;
 }
 
+template <bool NT, typename V>
+__device__ __forceinline__ V ld(const V* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+
 // The operands of one block of 32 keys as they come from memory.
 struct KVBlock {
   bf16x8 kw[WIDE ? 2 * NQ : 1];  // [tile t][i]
@@ -83,8 +90,11 @@ struct KVBlock {
 // COOP: the four waves of a workgroup share one tile and one key range and take its 32-key blocks in turn; their
 // results meet in LDS.  Decode is bound by the latency of a wave's chain of loads, so the chain is made four times
 // shorter without more work for the kernel that joins the ranges.
-template <int QT, bool PREFETCH, bool COOP>
-__global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
+// NT: keys and values are read with non-temporal loads.  That is faster once a step's keys and values no longer fit the
+// memory-side cache (6.1 against 5.7 TB/s at batch 64 and 3,072 keys) and slower below (5.7 against 6.1 TB/s at batch
+// 64 and 1,024 keys), so the kernel chooses by the number of keys the step reads, which the host leaves in the tiles.
+template <int QT, bool PREFETCH, bool COOP, bool NT>
+__device__ __forceinline__ void attn_tiles(const AttnParams& a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int G = a.heads / a.kv_heads;
@@ -192,10 +202,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
       const bf16_t* krow = kbase + (((size_t)page * kv_row) << psh) + (size_t)(key & pmask) * HD;
       if (WIDE) {
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) blk.kw[t * NQ + i] = *reinterpret_cast<const bf16x8*>(krow + i * 32);
+        for (int i = 0; i < NQ; ++i) blk.kw[t * NQ + i] = ld<NT>(reinterpret_cast<const bf16x8*>(krow + i * 32));
       } else {
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) blk.kn[t * NQ + i] = *reinterpret_cast<const s16x4*>(krow + i * 16);
+        for (int i = 0; i < NQ; ++i) blk.kn[t * NQ + i] = ld<NT>(reinterpret_cast<const s16x4*>(krow + i * 16));
       }
     }
   };
@@ -210,8 +220,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
     const bf16_t* v1 = vbase + (((size_t)page_of(k1) * kv_row) << psh) + (k1 & pmask);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      blk.v[dt][0] = *reinterpret_cast<const bf16x4*>(v0 + dt * v_step);
-      blk.v[dt][1] = *reinterpret_cast<const bf16x4*>(v1 + dt * v_step);
+      blk.v[dt][0] = ld<NT>(reinterpret_cast<const bf16x4*>(v0 + dt * v_step));
+      blk.v[dt][1] = ld<NT>(reinterpret_cast<const bf16x4*>(v1 + dt * v_step));
     }
   };
   auto load = [&](KVBlock& blk, int kb) {
@@ -394,6 +404,20 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
         a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum[u];
       }
     }
+  }
+}
+
+constexpr long NT_FROM_BYTES = 320L << 20;  // keys and values of a step (one layer) from which non-temporal loads pay
+
+template <int QT, bool PREFETCH, bool COOP>
+__global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
+  if constexpr (QT == 1) {
+    // decode tiles carry the number of keys that the step's decode rows read in all (the same in every tile)
+    const long bytes = (long)a.tiles[5] * a.kv_heads * HD * 4;
+    if (bytes >= NT_FROM_BYTES) attn_tiles<QT, PREFETCH, COOP, true>(a);
+    else attn_tiles<QT, PREFETCH, COOP, false>(a);
+  } else {
+    attn_tiles<QT, PREFETCH, COOP, false>(a);
   }
 }
 

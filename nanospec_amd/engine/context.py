@@ -141,6 +141,7 @@ def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, s
         req = np.nonzero(lens_a == 1)[0].astype(np.int32)
         d = np.zeros((len(req), TILE_INTS), dtype=np.int32)
         d[:, 0], d[:, 2], d[:, 3], d[:, 4] = req, indptr[req], 1, kv[req]
+        d[:, 5] = min(int(kv[req].sum()), 2**31 - 1)  # what the step's decode rows read in all: the kernel's choice of loads
         put("dtiles", d.reshape(-1))
     if layout.Tc:
         rows = [(b, t0, indptr[b], n, kv[b], 0, 0, 0) for b, n in enumerate(lens) if n != 1 for t0 in range(0, n, CHUNK_TILE)]

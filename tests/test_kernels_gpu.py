@@ -420,7 +420,7 @@ def test_attention_generic(dtype, case, heads, kvh, hd, page):
         assert ulps_of_row_max(out.cpu(), ref).max() <= 4  # the reference's bound, tests/test_backends.py:71
 
 
-def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False):
+def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0):
     n = sum(lens)
     indptr = [0]
     for l in lens:
@@ -430,6 +430,8 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
     tile = lambda b, t0: [b, t0, indptr[b], lens[b], starts[b] + lens[b], 0, 0, 0]
     ct = [tile(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16 * qt)]
     dt = [tile(b, 0) for b, l in enumerate(lens) if l == 1]
+    for t in dt:
+        t[5] = step_keys  # the keys all decode rows of the step read: from some number on the kernel reads them past the cache
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
     if ct:
         ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1, qt=qt)
@@ -459,8 +461,9 @@ def test_attention_mfma(case, heads, kvh, hd, page):
     n = sum(lens)
     q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
-    for splits, qt, coop in ((1, 2, False), (3, 1, False), (7, 2, True), (33, 1, False), (1, 1, True), (2, 2, True)):
-        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt, coop=coop)
+    for splits, qt, coop, step_keys in ((1, 2, False, 0), (3, 1, False, 0), (7, 2, True, 0), (33, 1, False, 2**30), (1, 1, True, 2**30),
+                                        (2, 2, True, 0)):
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt, coop=coop, step_keys=step_keys)
         u = ulps_of_row_max(out.cpu(), ref).max()
         assert u <= 4, f"{case} splits={splits} qt={qt} coop={coop}: {u:.2f} ulps"
 
