@@ -44,7 +44,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 // A tile descriptor, filled on the host: {request, first token of the tile among the request's tokens of this step
 // (tiles of one request follow each other every 16 qt / hp tokens),
 // row of the request's first token in the batch, tokens of the request in this step, keys after this step,
-// for decode tiles the keys that all decode rows of the step read together, 0, 0}.
+// for decode tiles the keys that all decode rows of the step read together over all layers, 0, 0}.
 struct AttnParams {
   bf16_t* out;        // [tokens, heads, HD]
   float* part_o;      // [n_tiles * (16 / hp) * heads, splits, HD]   (splits > 1)
@@ -90,9 +90,10 @@ struct KVBlock {
 // COOP: the four waves of a workgroup share one tile and one key range and take its 32-key blocks in turn; their
 // results meet in LDS.  Decode is bound by the latency of a wave's chain of loads, so the chain is made four times
 // shorter without more work for the kernel that joins the ranges.
-// NT: keys and values are read with non-temporal loads.  That is faster once a step's keys and values no longer fit the
-// memory-side cache (6.1 against 5.7 TB/s at batch 64 and 3,072 keys) and slower below (5.7 against 6.1 TB/s at batch
-// 64 and 1,024 keys), so the kernel chooses by the number of keys the step reads, which the host leaves in the tiles.
+// NT: keys and values are read with non-temporal loads.  A step reads every layer's keys and values once; if all of them
+// together fit the memory-side cache they are still there at the next step and plain loads find them, otherwise they only
+// push other data out and non-temporal loads are the faster ones (6.1 against 5.7 TB/s at batch 64 and 3,072 keys of the
+// 8B shape).  The kernel chooses by the number of keys over all layers, which the host leaves in the tiles.
 template <int QT, bool PREFETCH, bool COOP, bool NT>
 __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -407,12 +408,12 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
   }
 }
 
-constexpr long NT_FROM_BYTES = 320L << 20;  // keys and values of a step (one layer) from which non-temporal loads pay
+constexpr long NT_FROM_BYTES = 192L << 20;  // keys and values of a step (all layers) from which non-temporal loads pay
 
 template <int QT, bool PREFETCH, bool COOP>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   if constexpr (QT == 1) {
-    // decode tiles carry the number of keys that the step's decode rows read in all (the same in every tile)
+    // decode tiles carry the number of keys that the step's decode rows read over all layers (the same in every tile)
     const long bytes = (long)a.tiles[5] * a.kv_heads * HD * 4;
     if (bytes >= NT_FROM_BYTES) attn_tiles<QT, PREFETCH, COOP, true>(a);
     else attn_tiles<QT, PREFETCH, COOP, false>(a);

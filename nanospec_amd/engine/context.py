@@ -113,9 +113,11 @@ class StepContext:
         return plans
 
 
-def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, slots, want_rows, tables: list[np.ndarray]) -> None:
+def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, slots, want_rows, tables: list[np.ndarray],
+               kv_layers: int = 1) -> None:
     """Write one batch into ``host`` (int32, at least layout.total long).  ``starts``/``lens``: first
-    position and token count per request; ``tables[g]``: int32 [B, P] block tables."""
+    position and token count per request; ``tables[g]``: int32 [B, P] block tables; ``kv_layers``: how many layers keep
+    keys and values in pages."""
     f = layout.fields
     B = layout.B
     lens_a = np.asarray(lens, dtype=np.int32)
@@ -141,7 +143,9 @@ def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, s
         req = np.nonzero(lens_a == 1)[0].astype(np.int32)
         d = np.zeros((len(req), TILE_INTS), dtype=np.int32)
         d[:, 0], d[:, 2], d[:, 3], d[:, 4] = req, indptr[req], 1, kv[req]
-        d[:, 5] = min(int(kv[req].sum()), 2**31 - 1)  # what the step's decode rows read in all: the kernel's choice of loads
+        # keys the decode rows read in this step over all layers: what would have to stay cached until the next step, by
+        # which the attention kernel chooses its loads
+        d[:, 5] = min(int(kv[req].sum()) * kv_layers, 2**31 - 1)
         put("dtiles", d.reshape(-1))
     if layout.Tc:
         rows = [(b, t0, indptr[b], n, kv[b], 0, 0, 0) for b, n in enumerate(lens) if n != 1 for t0 in range(0, n, CHUNK_TILE)]

@@ -73,6 +73,7 @@ class ModelRunner:
         self.max_requests = max_requests
         self.stream = torch.cuda.Stream(device=self.device)
         self.arena = Arena(self.device)
+        self._kv_layers = sum(1 for need in model.cache_needs if need is not None and hasattr(need, "kv_heads"))
         self.link_norms = True  # see StepContext; set False before the first step to run every norm as a kernel of its own
         n_groups = len(manager.groups)
         # host mirror of every live request's block tables, one row per state slot
@@ -214,7 +215,7 @@ class ModelRunner:
             want_rows.extend(base + w for w in e.want)
             base += n
         tables = [t[slots, :width] for t in self._tables]
-        fill_batch(self._host.numpy(), layout, token_ids, starts, lens, slots, want_rows, tables)
+        fill_batch(self._host.numpy(), layout, token_ids, starts, lens, slots, want_rows, tables, self._kv_layers)
         if n_patch:
             first_row = np.concatenate(([0], np.cumsum(lens)[:-1]))
             self._put_patch(self._host.numpy(), layout, [int(first_row[e]) for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
@@ -251,7 +252,7 @@ class ModelRunner:
         token_ids = [e.tokens[0] for e in entries] + [0] * n_pad
         st = list(starts) + [0] * n_pad
         tables = [t[slots, :] for t in self._tables]
-        fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables)
+        fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables, self._kv_layers)
         if device_tokens:
             self._put_patch(g.host_np, g.layout, [e for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
         off, n = g.layout.fields["sample_opts"]
