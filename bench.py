@@ -47,34 +47,41 @@ def prefill_flops(c, n: int, rows_with_logits: int) -> float:
 
 
 def decode_run(model, cfg, batch: int, prompt_len: int, first_ctx: int, steps: int, warmup: int, block_size: int, seed: int):
-    """-> (seconds for ``steps`` decode steps, context at the first and after the last timed step)."""
+    """-> (seconds for ``steps`` decode steps, mean context of the first timed step and one past that of the last)."""
     import torch
 
     from nanospec_amd import Engine, EngineConfig, SamplingParams
 
-    total = first_ctx + warmup + steps + 1
+    # Prompts are taken in portions beside the decoding of the requests that are through theirs, so the first request is a
+    # few tokens ahead of the last when the clock starts.  No request ends before the clock stops: the engine enqueues
+    # each step one ahead of the one it waits for, so the step enqueued in the last warm-up call has run before the
+    # clock starts and the last timed call enqueues one more, and the clock covers the GPU's work of exactly ``steps`` steps.
+    ahead = batch * -(-first_ctx // 2048) + 2
+    total = first_ctx + ahead + warmup + steps + 2
     blocks = batch * -(-(total + 1) // block_size) + 2
     eng = Engine(model, EngineConfig(num_blocks=blocks, block_size=block_size, max_admit=batch, max_running=batch,
                                      max_step_tokens=2048, prefill_chunk=2048, max_seq_len=total + block_size))
     g = torch.Generator().manual_seed(seed)
     # a prompt of ``first_ctx`` tokens puts the first decode step at that context
     prompts = torch.randint(0, cfg.vocab_size, (batch, first_ctx), generator=g).tolist()
-    reqs = [eng.add(p, SamplingParams(max_tokens=warmup + steps + 1)) for p in prompts]
+    reqs = [eng.add(p, SamplingParams(max_tokens=total - first_ctx)) for p in prompts]
     while any(r.computed < first_ctx for r in reqs):
         eng.step()  # prefill in portions of at most 2,048 tokens
     for _ in range(warmup):
         eng.step()
     eng.runner.synchronize()
     torch.cuda.synchronize()
+    had = [len(r.out_tokens) for r in reqs]
+    ctx0 = sum(r.computed for r in reqs) / batch + 1  # keys that the first timed step of the GPU attends to, on average
     t0 = time.perf_counter()
     for _ in range(steps):
         eng.step()
     eng.runner.synchronize()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    assert all(len(r.out_tokens) == 1 + warmup + steps for r in reqs), "a decode step did not produce one token per request"
+    assert all(len(r.out_tokens) == n + steps for r, n in zip(reqs, had)), "a decode step did not produce one token per request"
+    assert all(r.computed == len(r.prompt_ids) + n + steps for r, n in zip(reqs, had)), "the step enqueued ahead is missing"
     assert eng.runner.last_used_graph, "decode steps did not replay a captured graph"
-    ctx0 = first_ctx + 1 + warmup
     del eng
     torch.cuda.empty_cache()
     return dt, ctx0, ctx0 + steps
@@ -147,7 +154,8 @@ def main() -> int:
     if not a.no_points:
         k = min(steps, 256)
         for b in (1, 64):
-            d, _, _ = decode_run(model, cfg, b, prompt, 3072 - k // 2 - a.warmup - 1, k, a.warmup, block, seed=2 + b)
+            lead = b  # the requests are b / 2 tokens into their decoding, on average, when the last is through its prompt
+            d, _, _ = decode_run(model, cfg, b, prompt, 3072 - k // 2 - a.warmup - 1 - lead, k, a.warmup, block, seed=2 + b)
             points[f"decode_b{b}"] = round(b * k / d, 1)
 
     line = {
@@ -158,8 +166,8 @@ def main() -> int:
         "config": {"model": "Llama-3.1-8B shape", "layers": shape["num_hidden_layers"], "layers_of_shape": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": prompt, "ctx_first_step": ctx0,
-                   "ctx_last_step": ctx1 - 1, "page_size": block, "parallelism": "single GPU", "graphs": True},
+                   "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": prompt, "ctx_first_step": round(ctx0, 1),
+                   "ctx_last_step": round(ctx1 - 1, 1), "page_size": block, "parallelism": "single GPU", "graphs": True},
         "prefill": {"value": round(p_tokens / p_dt, 1), "tokens": p_tokens, "ms": round(1000 * p_dt, 3), "frac": round(p_frac, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},

@@ -113,15 +113,16 @@ class Engine:
         the next step, whose input ids are taken on the GPU from this step's samples; only then does the host wait for
         this step's tokens.  The host's work between two steps is hidden behind the GPU's.  A request that turns out to
         have stopped on an end-of-sequence token has then already been given one more step, whose result is dropped."""
-        launched, self._ahead = self._ahead, None
-        if launched is None:
-            work = self.sched.next_batch()
-            if not work:
-                return []
-            launched = self._launch(work, None)
-        if self._may_look_ahead(launched):
-            self._ahead = self._launch_ahead(launched)
-        return self._harvest(launched)
+        with torch.cuda.stream(self.runner.stream):  # the whole step lives on the runner's stream: no waits between streams
+            launched, self._ahead = self._ahead, None
+            if launched is None:
+                work = self.sched.next_batch()
+                if not work:
+                    return []
+                launched = self._launch(work, None)
+            if self._may_look_ahead(launched):
+                self._ahead = self._launch_ahead(launched)
+            return self._harvest(launched)
 
     def _launch(self, work: list[Work], token_src) -> dict:
         """Enqueue one step and its sampling.  ``token_src``: the launched step whose samples are this step's input ids."""

@@ -154,8 +154,13 @@ class ModelRunner:
         for rc in rcs:
             self._mirror(rc)
         n_want = sum(len(e.want) for e in entries)
+        # A caller that works on another stream is ordered against this one on both sides.  A caller already on the
+        # runner's stream (the engine) needs neither wait, and a wait between streams before every replay of a captured
+        # step was measured to slow the replay itself by several per cent.
         caller = torch.cuda.current_stream(self.device)
-        self.stream.wait_stream(caller)  # whatever the caller still reads of the last step's results
+        foreign = caller != self.stream
+        if foreign:
+            self.stream.wait_stream(caller)  # whatever the caller still reads of the last step's results
         if self._staged is not None:
             self._staged.synchronize()  # the last batch has left the pinned staging buffers
         with torch.cuda.stream(self.stream):
@@ -165,7 +170,8 @@ class ModelRunner:
             else:
                 logits = self._step_eager(entries, rcs, starts, lens, n_want, device_tokens)
                 self.last_used_graph = False
-        caller.wait_stream(self.stream)  # the caller's stream sees the logits
+        if foreign:
+            caller.wait_stream(self.stream)  # the caller's stream sees the logits
         for e, rc in zip(entries, rcs):
             mgr.commit(e.req_id, len(e.tokens))
         return logits

@@ -277,6 +277,26 @@ def test_lookahead_changes_nothing_but_the_timing(tiny_folders, tmp_path):
     assert any(o[-1] in stops and len(o) < p.max_tokens for o, p in zip(outs[True], params)), "no request stopped on an end token"
 
 
+def test_engine_on_a_callers_side_stream(tiny_folders):
+    """The engine works on its runner's stream whatever stream the caller is on, hands the caller's stream back, and
+    its tokens are those of a run from the default stream."""
+    from nanospec_amd import SamplingParams
+
+    name = "A"
+    model = model_of(tiny_folders[name], name, torch.float32)
+    prompts = prompts_of(name)
+    params = [SamplingParams(max_tokens=NEW[name])] * len(prompts)
+    base, _, _ = run_engine(model, prompts, params, num_blocks=96, block_size=8)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        busy = torch.randn(1 << 20, device="cuda").cumsum(0)  # work of the caller's own, still under way
+        reqs, _, eng = run_engine(model, prompts, params, num_blocks=96, block_size=8)
+        assert torch.cuda.current_stream() == side
+    assert eng.runner.stream not in (side, torch.cuda.default_stream())
+    assert [r.out_tokens for r in reqs] == [r.out_tokens for r in base]
+    del busy
+
+
 def test_refuses_what_it_cannot_run(tiny_folders):
     from nanospec_amd import Engine, EngineConfig, SamplingParams
     from nanospec_amd.cache import PoolExhausted
