@@ -396,7 +396,7 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
         *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
       }
     } else {
-      const size_t pcol = ((size_t)tile * (16 / a.hp) + tt) * a.heads + head;
+      const size_t pcol = ((size_t)tile * (QT * 16 / a.hp) + tt) * a.heads + head;
       float* po = a.part_o + (pcol * a.splits + split) * HD;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[u][dt];
@@ -456,9 +456,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int G = a.heads / a.kv_heads;
     const int hblks = (G + 3) / 4;
     const int ny = a.kv_heads * hblks;
-    const int y = blockIdx.x % ny;
+    const int split = blockIdx.x % a.splits, ts = blockIdx.x / a.splits;  // the ranges of a tile start together
+    const int y = ts % ny;
     // tiles are listed in the order of the tokens; the last ones see the most keys, so they start first
-    const int tile = a.n_tiles - 1 - blockIdx.x / ny;
+    const int tile = a.n_tiles - 1 - ts / ny;
     const int kvh = y / hblks, hin = (y % hblks) * 4 + wave;
     const bool head_ok = hin < G;  // a wave without a head still fetches its share of the keys and values
     const int head = kvh * G + (head_ok ? hin : 0);
@@ -483,7 +484,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int wlo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
     const int full_hi = first_pos;                                                  // keys <= full_hi are seen by every token
     const int full_lo = a.window > 0 ? max(0, last_pos - a.window + 1) : 0;         // ... if they are >= full_lo
-    const int tile_kb0 = wlo / 32, tile_kb1 = (whi + 31) / 32;
+    int tile_kb0 = wlo / 32, tile_kb1 = (whi + 31) / 32;
+    if (a.splits > 1) {  // this workgroup's range of the tile's blocks; it may be empty
+      const int per = (tile_kb1 - tile_kb0 + a.splits - 1) / a.splits;
+      tile_kb0 = min(tile_kb1, tile_kb0 + split * per);
+      tile_kb1 = min(tile_kb1, tile_kb0 + per);
+    }
     const int steps = (tile_kb1 - tile_kb0 + 1) / 2;  // blocks of the first set; the second has as many or one fewer
     const int kb0 = half ? tile_kb0 + steps : tile_kb0, kb1 = half ? tile_kb1 : tile_kb0 + steps;
 
@@ -701,6 +707,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
       const float msafe = mstar == -INFINITY ? 0.f : mstar;
       const float w0 = fast_exp2((m[u] - msafe) * a.scale_log2), w1 = fast_exp2((m1 - msafe) * a.scale_log2);
       lsum[u] = lsum[u] * w0 + l1 * w1;
+      m[u] = mstar;  // what the sums now refer to: a range's maximum goes out with them
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(join + (u * DT + dt) * 4);
@@ -714,12 +721,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
       lsum[u] += __shfl_xor(lsum[u], 16, 64);
       lsum[u] += __shfl_xor(lsum[u], 32, 64);
       if (!col_ok[u]) continue;
-      const size_t col = (size_t)(q0 + t0 + u * 16 + c) * a.heads + head;
-      const float inv = 1.f / lsum[u];
+      // o[u][dt][j] is channel 16 dt + 4 g + j of column c
+      if (a.splits == 1) {
+        const size_t col = (size_t)(q0 + t0 + u * 16 + c) * a.heads + head;
+        const float inv = 1.f / lsum[u];
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {  // o[u][dt][j] is channel 16 dt + 4 g + j of column c
-        bf16x4 r = {(bf16_t)(o[u][dt][0] * inv), (bf16_t)(o[u][dt][1] * inv), (bf16_t)(o[u][dt][2] * inv), (bf16_t)(o[u][dt][3] * inv)};
-        *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
+        for (int dt = 0; dt < DT; ++dt) {
+          bf16x4 r = {(bf16_t)(o[u][dt][0] * inv), (bf16_t)(o[u][dt][1] * inv), (bf16_t)(o[u][dt][2] * inv), (bf16_t)(o[u][dt][3] * inv)};
+          *reinterpret_cast<bf16x4*>(a.out + col * HD + dt * 16 + g * 4) = r;
+        }
+      } else {  // as the ranges of a decode tile: unnormalised sums, maximum in the exponent's units, total
+        const size_t pcol = ((size_t)tile * 32 + u * 16 + c) * a.heads + head;
+        float* po = a.part_o + (pcol * a.splits + split) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[u][dt];
+        if (g == 0) {
+          a.part_ml[(pcol * a.splits + split) * 2] = m[u] * a.scale_log2;
+          a.part_ml[(pcol * a.splits + split) * 2 + 1] = lsum[u];
+        }
       }
     }
   }
@@ -731,10 +750,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
 // results are addressed by tile, so nothing here waits for the tile descriptor except the final store.
 __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                                          const float* __restrict__ part_ml, const int* __restrict__ tiles,
-                                                         int heads, int hp, int splits) {
+                                                         int heads, int tile_tokens, int splits) {
   const int tile = blockIdx.x, head = blockIdx.y, tt = blockIdx.z;
   const int lane = threadIdx.x;
-  const size_t pcol = ((size_t)tile * (16 / hp) + tt) * heads + head;
+  const size_t pcol = ((size_t)tile * tile_tokens + tt) * heads + head;
   const float* ml = part_ml + pcol * splits * 2;
   float ms = -INFINITY, ls = 0.f;
   if (lane < splits) {
@@ -784,7 +803,8 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ ou
 extern "C" int ns_attn_mfma_head_dim() { return HD; }
 extern "C" int ns_attn_mfma_page_size() { return PS; }
 
-// Workspace, when splits > 1: part_o holds n_tiles*(16/hp)*heads*splits*HD floats, part_ml n_tiles*(16/hp)*heads*splits*2.
+// Workspace, when splits > 1: with T = qt*16/hp tokens in a tile, part_o holds n_tiles*T*heads*splits*HD floats and
+// part_ml n_tiles*T*heads*splits*2.
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
@@ -795,7 +815,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
   if (!(scale > 0.f)) return NS_ERR_BAD_ARG;  // maxima are tracked on unscaled scores
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
-  if (qt != 1 && !(qt == 2 && hp == 1 && splits == 1 && !coop)) return NS_ERR_BAD_ARG;
+  if (qt != 1 && !(qt == 2 && hp == 1 && !coop)) return NS_ERR_BAD_ARG;
   AttnParams a;
   a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
   a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
@@ -808,7 +828,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const long blocks = coop ? items : (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
   if (qt == 2 && SHARED_OK) {
-    const long wgs = (long)n_tiles * kv_heads * ((G + 3) / 4);
+    const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
     attn_prefill_kernel<<<(unsigned)wgs, 512, 0, stream>>>(a);
   } else if (qt == 2)
@@ -820,7 +840,8 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const int st = ns_launch_status();
   if (st != NS_OK || splits == 1) return st;
   if (heads > 65535) return NS_ERR_BAD_ARG;
-  attn_reduce_kernel<<<dim3(n_tiles, heads, 16 / hp), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml,
-                                                                      tiles, heads, hp, splits);
+  const int tile_tokens = qt * 16 / hp;
+  attn_reduce_kernel<<<dim3(n_tiles, heads, tile_tokens), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml,
+                                                                           tiles, heads, tile_tokens, splits);
   return ns_launch_status();
 }

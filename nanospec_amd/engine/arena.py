@@ -13,12 +13,14 @@ import math
 import torch
 
 _ALIGN = 256
+_ESIZE: dict = {}  # bytes per element of the types asked for so far
 
 
 class Arena:
     def __init__(self, device, nbytes: int = 0, fixed: bool = False) -> None:
         self.device, self.fixed = device, fixed
         self._chunks: list[torch.Tensor] = []
+        self._typed: dict = {}  # (chunk, dtype) -> the chunk seen as that type
         self._cur, self._off = -1, 0
         self._high = 0  # bytes one step needed at most, over all chunks
         if nbytes:
@@ -27,7 +29,9 @@ class Arena:
 
     def take(self, shape, dtype) -> torch.Tensor:
         shape = tuple(int(s) for s in shape)
-        nbytes = max(1, math.prod(shape)) * torch.empty(0, dtype=dtype).element_size()
+        esize = _ESIZE.get(dtype) or _ESIZE.setdefault(dtype, torch.empty(0, dtype=dtype).element_size())
+        count = math.prod(shape)
+        nbytes = max(1, count) * esize
         need = -(-nbytes // _ALIGN) * _ALIGN
         while self._cur < 0 or self._off + need > self._chunks[self._cur].numel():
             if self._cur + 1 < len(self._chunks):
@@ -38,8 +42,14 @@ class Arena:
             size = max(need, 2 * sum(c.numel() for c in self._chunks), 1 << 20)
             self._chunks.append(torch.empty(size, dtype=torch.uint8, device=self.device))
             self._cur, self._off = len(self._chunks) - 1, 0
-        chunk = self._chunks[self._cur]
-        out = chunk[self._off : self._off + nbytes].view(dtype).view(shape)
+        # a view of the chunk in the wanted type is kept, so a buffer costs one slice and one reshape (offsets are
+        # multiples of 256 bytes, hence of every element size)
+        typed = self._typed.get((self._cur, dtype))
+        if typed is None:
+            chunk = self._chunks[self._cur]
+            typed = self._typed[self._cur, dtype] = chunk[: chunk.numel() // esize * esize].view(dtype)
+        first = self._off // esize
+        out = typed[first : first + count].view(shape)
         self._off += need
         return out
 
@@ -54,4 +64,5 @@ class Arena:
         if len(self._chunks) > 1 and not self.fixed:
             total = sum(c.numel() for c in self._chunks)
             self._chunks = [torch.empty(total, dtype=torch.uint8, device=self.device)]
+            self._typed.clear()
         self._cur, self._off = (0, 0) if self._chunks else (-1, 0)

@@ -25,6 +25,8 @@ import numpy as np
 import torch
 
 CHUNK_TILE = 32  # tokens per attention tile of a prompt portion (two 16-column tiles per wave)
+CHUNK_RANGE_BLOCKS = 16  # the fewest 32-key blocks that a range of a prompt portion's keys is worth a workgroup of its own
+CHUNK_FILL = 256  # workgroups of prompt-portion tiles (one fits a compute unit) below which their keys are cut into ranges
 TILE_INTS = 8  # a tile descriptor: request, first token, row of the request's first token, tokens, keys, 0, 0, 0
 
 
@@ -67,8 +69,10 @@ class StepContext:
     """Device views of one step's batch plus the arena; handed to every part."""
 
     def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, fixed_splits: bool = False,
-                 link_norms: bool = True) -> None:
+                 link_norms: bool = True, max_chunk_kv: int | None = None) -> None:
         self.layout, self.arena = layout, arena
+        # the most keys that a request bringing a prompt portion has after this step (at most max_kv_len)
+        self.max_chunk_kv = max_kv_len if max_chunk_kv is None else max_chunk_kv
         # blocks may let the products around an RMS norm do the norm's work (see parts.block.PreNormBlock.forward)
         self.link_norms = link_norms
         self.n_tokens, self.n_reqs = layout.N, layout.B
@@ -89,12 +93,20 @@ class StepContext:
 
     def attention_plans(self, group: int, kv_heads: int, head_dim: int) -> list[AttentionPlan]:
         """How the matrix-core attention kernel is launched for a mixer with ``group`` query heads per
-        key/value head: prompt portions as 32-token tiles of one head; decode rows with all heads of a
+        key/value head: prompt portions as 32-token tiles of one head, their keys cut into ranges when there are too few
+        tiles to fill the GPU and many keys (a short portion late in a long prompt); decode rows with all heads of a
         group in one tile and the keys cut into ranges so that the launch fills the GPU."""
         plans = []  # made afresh per call: the workspace lives in the caller's arena scope
         lay = self.layout
         if lay.Tc:
-            plans.append(AttentionPlan(self._ctiles, 1, 1, None, qt=CHUNK_TILE // 16))
+            wgs = lay.Tc * kv_heads * -(-group // 4)
+            blocks = -(-self.max_chunk_kv // 32)
+            splits = max(1, min(16, CHUNK_FILL // wgs, blocks // CHUNK_RANGE_BLOCKS))
+            ws = None
+            if splits > 1:
+                cols = lay.Tc * CHUNK_TILE * kv_heads * group
+                ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
+            plans.append(AttentionPlan(self._ctiles, 1, splits, ws, qt=CHUNK_TILE // 16))
         if lay.Td:
             hp = 1
             while hp < min(group, 16):

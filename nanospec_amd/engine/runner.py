@@ -231,7 +231,9 @@ class ModelRunner:
         if n_patch:
             self._apply_patch(self._dev, layout, device_tokens[0], n_patch)
         self.arena.reset()
-        ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv, link_norms=self.link_norms)
+        chunk_kv = max((s + n for s, n in zip(starts, lens) if n != 1), default=0)
+        ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv, link_norms=self.link_norms,
+                          max_chunk_kv=chunk_kv)
         resid, delta = self.model.forward_hidden(ctx, self.storage.views)
         if not n_want:
             return None

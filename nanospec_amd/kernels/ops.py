@@ -33,7 +33,14 @@ def _ptr(t):
     return c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)  # the handle without building a Stream object
+_device_index = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """The current stream's handle; asked for at every launch, so by the shortest way that torch offers."""
+    if _raw_stream is not None and _device_index is not None:
+        return c_void_p(_raw_stream(_device_index()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -482,7 +489,7 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     """bfloat16 attention on the matrix cores for the tiles described in ``tiles`` (int32 [n_tiles, 8]: request, first
     token of the tile among the request's tokens of this step, row of the request's first token in ``q``, tokens of the
     request in this step, keys after this step, three zeros).  ``hp`` heads of a group times 16/hp tokens make a tile;
-    with ``qt`` = 2 (only with hp = 1 and no splits) a tile is 32 tokens.  ``splits`` > 1 cuts the keys of every tile
+    with ``qt`` = 2 (only with hp = 1) a tile is 32 tokens.  ``splits`` > 1 cuts the keys of every tile
     into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors.  With ``coop`` the four
     waves of a workgroup share each tile and range (for decode, where a wave's chain of loads is what takes the time)."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
@@ -495,15 +502,15 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
         raise KernelRefused(f"attention_mfma: tiles must be int32 [n_tiles, {TILE_INTS}], 16-byte aligned")
     if hp not in (1, 2, 4, 8, 16):
         raise KernelRefused("attention_mfma: hp is a power of two up to 16")
-    if qt != 1 and not (qt == 2 and hp == 1 and splits == 1 and not coop):
-        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1, no splits and no cooperating waves")
+    if qt != 1 and not (qt == 2 and hp == 1 and not coop):
+        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1 and no cooperating waves")
     n_tiles = tiles.shape[0]
     po = pm = None
     if splits > 1:
         if workspace is None or splits > 64:
             raise KernelRefused("attention_mfma: 2 to 64 key ranges are taken, with a workspace")
         po, pm = workspace
-        cols = n_tiles * (16 // hp) * heads
+        cols = n_tiles * (qt * 16 // hp) * heads
         if po.dtype != torch.float32 or pm.dtype != torch.float32 or po.numel() < cols * splits * head_dim or pm.numel() < cols * splits * 2:
             raise KernelRefused("attention_mfma: workspace too small")
     lib = build.attn(head_dim, page)

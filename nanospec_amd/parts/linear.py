@@ -61,6 +61,7 @@ class LinearWeight:
         fast = w.dtype == torch.bfloat16 and self.k % 8 == 0
         self.tiled = ops.TiledWeight(w) if (fast and tiled) else None
         self.plain = w if (keep_plain or self.tiled is None) else None
+        self._plain_t = self.plain.t() if self.plain is not None else None  # the library product's operand, made once
 
     def links_norms(self, rows: int) -> bool:
         """Whether a product of ``rows`` rows can take a ``PreNormed`` input and can end in the residual stream."""
@@ -109,7 +110,7 @@ class LinearWeight:
         if self.plain is not None and (not out_f32 or self.tiled is None):
             if out_f32:
                 return ops.linear_generic(x, self.plain, out=out, out_f32=True)
-            return torch.matmul(x, self.plain.t()) if out is None else torch.matmul(x, self.plain.t(), out=out)
+            return torch.matmul(x, self._plain_t) if out is None else torch.matmul(x, self._plain_t, out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
         ksplit, nt = ops.wide_plan(self.n, self.k)
@@ -133,6 +134,7 @@ class GatedWeights:
         fast = gate.dtype == torch.bfloat16 and self.k % 8 == 0
         self.tiled = (ops.TiledWeight(gate), ops.TiledWeight(up)) if fast else None
         self.stacked = torch.cat([gate, up]) if (keep_plain or not fast) else None  # [2 I, K] for the two-kernel path
+        self._stacked_t = self.stacked.t() if self.stacked is not None else None
 
     def links_norms(self, rows: int) -> bool:
         return self.tiled is not None and rows <= STREAM_ROWS
@@ -157,5 +159,5 @@ class GatedWeights:
         if self.dtype == torch.float32 or self.k % 8:
             ops.linear_generic(x, self.stacked, out=gu)
         else:
-            torch.matmul(x, self.stacked.t(), out=gu)
+            torch.matmul(x, self._stacked_t, out=gu)
         return ops.silu_mul(gu, out=out)

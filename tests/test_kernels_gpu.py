@@ -420,7 +420,8 @@ def test_attention_generic(dtype, case, heads, kvh, hd, page):
         assert ulps_of_row_max(out.cpu(), ref).max() <= 4  # the reference's bound, tests/test_backends.py:71
 
 
-def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0):
+def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0,
+              chunk_splits=1):
     n = sum(lens)
     indptr = [0]
     for l in lens:
@@ -434,7 +435,12 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
         t[5] = step_keys  # the keys all decode rows of the step read: from some number on the kernel reads them past the cache
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
     if ct:
-        ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1, splits=1, qt=qt)
+        cols = len(ct) * 16 * qt * heads
+        ws = None
+        if chunk_splits > 1:  # filled with NaN: a range that is read without having been written shows
+            ws = (torch.full((cols * chunk_splits * hd,), float("nan"), device=DEV), torch.full((cols * chunk_splits * 2,), float("nan"), device=DEV))
+        ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1,
+                           splits=chunk_splits, workspace=ws, qt=qt)
     if dt:
         hp = 1
         while hp < min(group, 16):
@@ -461,11 +467,13 @@ def test_attention_mfma(case, heads, kvh, hd, page):
     n = sum(lens)
     q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
-    for splits, qt, coop, step_keys in ((1, 2, False, 0), (3, 1, False, 0), (7, 2, True, 0), (33, 1, False, 2**30), (1, 1, True, 2**30),
-                                        (2, 2, True, 0)):
-        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt, coop=coop, step_keys=step_keys)
+    # the last number: ranges that the keys of a prompt portion's tiles are cut into (16: more than most tiles have blocks)
+    for splits, qt, coop, step_keys, chunk_splits in ((1, 2, False, 0, 1), (3, 1, False, 0, 2), (7, 2, True, 0, 3), (33, 1, False, 2**30, 1),
+                                                      (1, 1, True, 2**30, 5), (2, 2, True, 0, 16)):
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt, coop=coop, step_keys=step_keys,
+                        chunk_splits=chunk_splits)
         u = ulps_of_row_max(out.cpu(), ref).max()
-        assert u <= 4, f"{case} splits={splits} qt={qt} coop={coop}: {u:.2f} ulps"
+        assert u <= 4, f"{case} splits={splits} qt={qt} coop={coop} chunk_splits={chunk_splits}: {u:.2f} ulps"
 
 
 @pytest.mark.parametrize("kernel", ["generic", "mfma"])
@@ -518,6 +526,8 @@ def test_attention_window(kernel, window):
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads, window=window).reshape(n, -1)
     if kernel == "mfma":
         out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=window)
+        cut = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=window, chunk_splits=3)
+        assert ulps_of_row_max(cut.cpu(), ref).max() <= 4
     else:
         positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
         token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)

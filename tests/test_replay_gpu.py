@@ -169,6 +169,37 @@ def test_norms_as_kernels_of_their_own(tiny_folders, name, schedule):
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("schedule", ["portions", "mixed"])
+def test_prompt_portions_with_their_keys_cut_into_ranges(tiny_folders, name, schedule, monkeypatch):
+    """A short portion late in a long prompt has its keys cut into ranges that workgroups of their own walk.  The tiny
+    models' prompts are too short for that by the engine's own rule, so the rule's threshold is lowered to one block."""
+    from nanospec_amd.engine import context
+    from nanospec_amd.kernels import ops
+
+    monkeypatch.setattr(context, "CHUNK_RANGE_BLOCKS", 1)
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, torch.bfloat16)
+    model = engine_model(folder, name, torch.bfloat16)
+    if schedule == "portions":
+        steps, where = traces.portions(seqs, seed=3)
+        max_tokens = 256
+    else:
+        steps, where, max_tokens = traces.mixed(seqs, seed=23)
+    cut = []
+    real = ops.attention_mfma
+
+    def counted(*a, **k):
+        if k.get("qt") == 2 and k.get("splits", 1) > 1:
+            cut.append(k["splits"])
+        return real(*a, **k)
+
+    monkeypatch.setattr(ops, "attention_mfma", counted)
+    replay(model, steps, where, ref, torch.bfloat16, max_tokens, page, graphs=False)
+    assert cut and max(cut) >= 3, "no portion had its keys cut into ranges"
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
 def test_one_weight_layout_only(tiny_folders, name):
     """Without the plain layout (models that fill the memory) steps of many tokens run in slices through the streaming
     kernels: same logits."""
