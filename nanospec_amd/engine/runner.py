@@ -23,7 +23,7 @@ from ..kernels import ops
 from .arena import Arena
 from .context import BatchLayout, StepContext, count_tiles, fill_batch
 
-GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64)  # reference: engine/graphs.py:22
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)  # reference: engine/graphs.py:22 (which stops at 64)
 PAD_REQUEST = "__pad__"
 
 

@@ -277,6 +277,25 @@ def test_lookahead_changes_nothing_but_the_timing(tiny_folders, tmp_path):
     assert any(o[-1] in stops and len(o) < p.max_tokens for o, p in zip(outs[True], params)), "no request stopped on an end token"
 
 
+def test_seventy_requests_decode_through_one_graph(tiny_folders):
+    """More rows than the reference's largest captured batch (64): the bucket of 128 rows, with pad rows, against the
+    same run without graphs."""
+    from nanospec_amd import SamplingParams
+
+    name = "B"
+    model = model_of(tiny_folders[name], name, torch.bfloat16)
+    vocab = TINY[name]["cfg"]["vocab_size"]
+    prompts = [random_tokens(3 + i % 11, vocab, 900 + i) for i in range(70)]
+    params = [SamplingParams(max_tokens=12 + i % 3) for i in range(70)]
+    outs = {}
+    for graphs in (True, False):
+        reqs, _, eng = run_engine(model, prompts, params, num_blocks=400, block_size=8, max_admit=70, max_running=70, cuda_graphs=graphs)
+        outs[graphs] = [r.out_tokens for r in reqs]
+        if graphs:
+            assert 128 in eng.runner._graphs, "the 70 rows did not replay the graph of 128"
+    assert outs[True] == outs[False]
+
+
 def test_engine_on_a_callers_side_stream(tiny_folders):
     """The engine works on its runner's stream whatever stream the caller is on, hands the caller's stream back, and
     its tokens are those of a run from the default stream."""
