@@ -32,16 +32,17 @@ class Replayer:
         self.runner = ModelRunner(model, self.manager, self.storage, slots, pages, use_graphs=use_graphs)
 
     def step(self, entries: list[dict], end: list) -> torch.Tensor | None:
-        batch = []
-        for e in entries:
-            if e["id"] not in self.manager:
-                self.runner.admit(e["id"])
-            batch.append(StepEntry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
-        logits = self.runner.step(batch)
-        out = logits.cpu() if logits is not None else None  # copied before anything is given back
-        for rid in end:
-            if rid in self.manager:
-                self.runner.release(rid)
+        with torch.cuda.stream(self.runner.stream):  # as the engine: everything on the runner's stream
+            batch = []
+            for e in entries:
+                if e["id"] not in self.manager:
+                    self.runner.admit(e["id"])
+                batch.append(StepEntry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+            logits = self.runner.step(batch)
+            out = logits.cpu() if logits is not None else None  # copied before anything is given back
+            for rid in end:
+                if rid in self.manager:
+                    self.runner.release(rid)
         return out
 
 
