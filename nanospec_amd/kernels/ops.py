@@ -280,6 +280,11 @@ class PreNormed:
         self.shape, self.dtype = x.shape, x.dtype
 
 
+class Added:
+    """What a part returns instead of its output when it has already added that output to the residual stream in place
+    (a library product with the stream as its addend): nothing is left to add and no statistics come with it."""
+
+
 def _prenorm_args(pre: "PreNormed | None", m: int, what: str):
     if pre is None:
         return c_void_p(None), c_int(0), c_int(0), c_float(0.0)

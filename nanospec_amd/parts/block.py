@@ -46,9 +46,9 @@ class PreNormBlock:
     links_blocks = True  # forward takes next_norm, next_sums and next_carry
 
     def forward(self, ctx, resid, delta, cache, owns_cache, delta_out, next_norm=None, next_sums=None, next_carry=None):
-        """``delta``: what the block before left to be added: a tensor (None at the start), a ``PartialSums``, or a
+        """``delta``: what the block before left to be added: a tensor (None at the start), a ``PartialSums``, a
         ``PreNormed``, in which case ``resid`` is already whole and the first norm's input comes ready for a product that
-        ``links_norms``.  ``next_norm``: the norm that will read this block's result (the next block's first one), if it
+        ``links_norms``, or an ``Added`` (``resid`` is whole, nothing else comes with it).  ``next_norm``: the norm that will read this block's result (the next block's first one), if it
         ``links_products``; ``next_sums`` (float32 [tokens, ceil(width / 16)]) and ``next_carry`` (float32, 16 * tokens *
         width, or None): buffers that live as long as the step.
         -> None, with the block's not yet added output in ``delta_out``; or that output in one of the forms of
@@ -62,8 +62,9 @@ class PreNormBlock:
         buf = lambda: ctx.arena.take(resid.shape, resid.dtype)
 
         # first norm and mixer
-        if isinstance(delta, ops.PreNormed):
-            h = delta if takes(self.mixer) else self.mixer_norm.forward(ctx, resid=resid, out=buf())
+        whole = (ops.PreNormed, ops.Added)  # forms in which resid already holds the sum
+        if isinstance(delta, whole):
+            h = delta if isinstance(delta, ops.PreNormed) and takes(self.mixer) else self.mixer_norm.forward(ctx, resid=resid, out=buf())
         else:
             h = self.mixer_norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None, out=buf())
         if ends(self.mixer) and lp(self.ffn_norm):
@@ -72,8 +73,8 @@ class PreNormBlock:
             a = self.mixer.forward(ctx, h, cache, owns_cache, out=buf())
 
         # second norm and feed-forward
-        if isinstance(a, ops.PreNormed):
-            h2 = a if takes(self.ffn) else self.ffn_norm.forward(ctx, resid=resid, out=buf())
+        if isinstance(a, whole):
+            h2 = a if isinstance(a, ops.PreNormed) and takes(self.ffn) else self.ffn_norm.forward(ctx, resid=resid, out=buf())
         else:
             h2 = self.ffn_norm.forward(ctx, resid=resid, x=a, write_resid=True, out=buf())
         if ends(self.ffn) and lp(next_norm) and next_sums is not None:

@@ -39,6 +39,8 @@ class IntoResidual:
         (at most 16 rows: the product's epilogue did the sum and the norm's statistics);
       * ``kernels.ops.PartialSums``: the ranges of a product whose K was cut, which the norm kernel adds up as it reads
         them (17 to 64 rows);
+      * ``kernels.ops.Added``: ``resid += output`` has been done in place by the product itself (more than 64 rows, through
+        the library), the norm still has its kernel;
       * a tensor: the output, still to be added by the norm kernel.
     ``next_weight``, ``eps``: that norm's weight and epsilon.  ``x_next`` (like resid), ``ssq`` (float32 [rows,
     ceil(width / 16)]) and ``carry`` (float32, 16 * rows * width): where the results go if they must outlive the block's
@@ -68,7 +70,7 @@ class LinearWeight:
         return self.tiled is not None and rows <= STREAM_ROWS
 
     def into_residual(self, x: torch.Tensor, link: IntoResidual, arena=None):
-        """x @ W^T on its way into the residual stream, in one of the three forms ``IntoResidual`` names."""
+        """x @ W^T on its way into the residual stream, in one of the forms ``IntoResidual`` names."""
         m = x.shape[0]
         take = (lambda shape, dtype: arena.take(shape, dtype)) if arena is not None else (lambda shape, dtype: torch.empty(shape, dtype=dtype, device=x.device))
         if self.links_norms(m) and x.dtype == torch.bfloat16 and ops.tiled_takes(x[:1], self.k):
@@ -86,6 +88,13 @@ class LinearWeight:
                 ws = take((need,), torch.float32)
             if ws is not None:
                 return ops.linear_wide(x, self.tiled, workspace=ws, ksplit=ksplit, nt=nt, defer=True)
+        r = link.resid
+        if (m > ops.SKINNY_MAX_ROWS and self._plain_t is not None and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16
+                and r.shape == (m, self.n) and r.is_contiguous()):
+            # many rows: the library's product takes the stream as its addend, resid = resid + x @ W^T summed in 32-bit and
+            # rounded once, so the norm after it reads one tensor instead of two and writes one instead of two
+            r.addmm_(x, self._plain_t)
+            return ops.Added()
         out = link.x_next if link.x_next is not None else take((m, self.n), x.dtype)
         return self(x, out=out, arena=arena)
 

@@ -102,7 +102,7 @@ class DecoderModel:
                 out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta, next_norm=nxt, next_sums=sums,
                                     next_carry=carry)
             else:
-                if isinstance(pending, ops.PreNormed):
+                if isinstance(pending, (ops.PreNormed, ops.Added)):
                     pending = None  # resid is whole already; a block that does not know the hand-over starts from it
                 elif isinstance(pending, ops.PartialSums):
                     pending = ops.reduce_partial(pending, out=delta)

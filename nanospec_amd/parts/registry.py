@@ -24,7 +24,7 @@ What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are 
 
 Optional, for parts whose products can do the work of the RMS norms around them (``parts.linear.IntoResidual``):
   norm         links_products = True, weight, spec.eps
-  mixer, ffn   ends_in_residual = True: forward(..., residual=IntoResidual) -> PreNormed | PartialSums | tensor;
+  mixer, ffn   ends_in_residual = True: forward(..., residual=IntoResidual) -> PreNormed | PartialSums | Added | tensor;
                links_norms(rows) -> bool: x may be a PreNormed
   block        links_blocks = True; forward(..., next_norm=None, next_sums=None, next_carry=None) -> None or one of
                those three
