@@ -426,17 +426,20 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 // Prompt portions when the head size is a multiple of 32 up to 128 and a page holds 8 tokens or more: a workgroup owns 32 tokens
 // of up to four query heads of one key/value head, one head per wave.  The four waves need the same keys and values,
 // so each block of 32 keys is fetched once per workgroup, a quarter by each wave, and handed round through LDS;
-// the next block is on its way from memory (and its page ids one block further ahead) while this one is used.
+// the next two blocks are on their way from memory (and the page ids one block further ahead) while this one is used.
 // A tile's keys are walked by two such sets of four waves at once, each taking half of the blocks; their results are
 // joined in LDS at the end.  The longest tiles set the time of a causal prompt, and this halves their chain of blocks.
 //   keys in LDS:   row 16 t + 4 a + b holds key 8 a + 4 t + b of the block, so that the scores a lane gets from the
 //                  two 16-key products are those of keys 8 g .. 8 g + 7: the order in which it then needs the values
 //   values in LDS: [channel][32 keys], as the pages hold them
-// Rows are padded by 16 bytes, which spreads the 16 rows of one load over all banks.
+// Rows are padded by 32 bytes.  A 16-byte LDS read is served for lanes 0-7 and 16-23 together (then 8-15 and 24-31, ...),
+// i.e. for eight rows at two neighbouring 16-byte columns: with rows of 2 HD + 32 and 96 bytes these sixteen pieces fall
+// into sixteen different groups of four banks (the bank-conflict counter reads zero; with 16 bytes of padding every read
+// took twice as long).
 // ------------------------------------------------------------------------------------------------
 constexpr bool SHARED_OK = WIDE && PS >= 8 && HD <= 128;  // larger heads do not fit two waves' registers per SIMD
-constexpr int KROW = HD + 8;               // elements of a key's row in LDS
-constexpr int VROW = 32 + 8;               // elements of a channel's row in LDS
+constexpr int KROW = HD + 16;               // elements of a key's row in LDS
+constexpr int VROW = 32 + 16;               // elements of a channel's row in LDS
 constexpr int CHUNKS = 32 * HD / 8;        // 16-byte pieces of a block's keys; as many of its values
 constexpr int PER_THREAD = (CHUNKS + 255) / 256;
 constexpr int CPR = PS / 8 < 4 ? PS / 8 : 4;  // 16-byte pieces of a block that lie side by side in a channel's row of a page
@@ -548,10 +551,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
       v_const[r] = (int)k_head + (v_ch[r] << psh) + ((v_kq[r] * 8) & pmask);
     }
     auto inside = [&](int kb) { return EVEN && kb * 32 >= wlo && kb * 32 + 31 < whi; };
-    int kp[PER_THREAD], vp[PER_THREAD];
-    bf16x8 kst[PER_THREAD], vst[PER_THREAD];
+    // Two blocks are on their way from memory at a time (a block's compute is shorter than the latency of its loads):
+    // register set (kb - kb0) & 1 holds block kb between its loads and its copy into LDS, and the page ids of block kb
+    // from a round before its loads.  Loads return in the order of issue, so a round asks for the next page ids before
+    // it asks for keys and values: waiting for those page ids a round later then leaves the keys and values in flight.
+    int kps[2][PER_THREAD], vps[2][PER_THREAD];
+    bf16x8 kst[2][PER_THREAD], vst[2][PER_THREAD];
     // Otherwise addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
-    auto fetch_pages = [&](int kb) {
+    auto fetch_pages = [&](int(&kp)[PER_THREAD], int(&vp)[PER_THREAD], int kb) {
       if (inside(kb)) {
         const int* row = table + kb * PPB;
 #pragma unroll
@@ -567,53 +574,56 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
         }
       }
     };
-    auto fetch = [&](int kb) {
+    auto fetch = [&](bf16x8(&kr)[PER_THREAD], bf16x8(&vr)[PER_THREAD], const int(&kp)[PER_THREAD], const int(&vp)[PER_THREAD], int kb) {
       if (inside(kb)) {
 #pragma unroll
         for (int r = 0; r < PER_THREAD; ++r) {
-          kst[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp[r] * kv_page + k_const[r]);
-          vst[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp[r] * kv_page + v_const[r]);
+          kr[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp[r] * kv_page + k_const[r]);
+          vr[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp[r] * kv_page + v_const[r]);
         }
       } else {
 #pragma unroll
         for (int r = 0; r < PER_THREAD; ++r) {
           const int key = min(max(kb * 32 + k_key[r], wlo), whi - 1);
-          kst[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp[r] * kv_page + k_head + (size_t)(key & pmask) * HD + k_off[r]);
+          kr[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp[r] * kv_page + k_head + (size_t)(key & pmask) * HD + k_off[r]);
           const int key8 = min(max(kb * 32 + v_kq[r] * 8, vlo), vhi);
-          vst[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp[r] * kv_page + k_head + ((size_t)v_ch[r] << psh) + (key8 & pmask));
+          vr[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp[r] * kv_page + k_head + ((size_t)v_ch[r] << psh) + (key8 & pmask));
         }
       }
     };
-    auto put = [&](int buf) {
+    auto put = [&](const bf16x8(&kr)[PER_THREAD], const bf16x8(&vr)[PER_THREAD], int buf) {
 #pragma unroll
       for (int r = 0; r < PER_THREAD; ++r)
         if (mine[r]) {
-          *reinterpret_cast<bf16x8*>(&lk[buf][k_lds[r]]) = kst[r];
-          *reinterpret_cast<bf16x8*>(&lv[buf][v_lds[r]]) = vst[r];
+          *reinterpret_cast<bf16x8*>(&lk[buf][k_lds[r]]) = kr[r];
+          *reinterpret_cast<bf16x8*>(&lv[buf][v_lds[r]]) = vr[r];
         }
     };
 
+    // One block of 32 keys for this wave's two 16-token columns.  The order of the source is the order of issue: the
+    // matrix instructions of one column run while the vector unit does the soft-max arithmetic of the other
+    // (scores u0, scores u1 | soft-max u0 under them, sums u0 | soft-max u1 under them, sums u1).
     auto block = [&](int buf, int kb) {
       const int key_base = kb * 32;
+      bf16x8 kf[2][NQ];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) kf[t][i] = *reinterpret_cast<const bf16x8*>(&lk[buf][(16 * t + c) * KROW + 32 * i + 8 * g]);
       f32x4 s[2][2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        bf16x8 kf[NQ];
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) kf[i] = *reinterpret_cast<const bf16x8*>(&lk[buf][(16 * t + c) * KROW + 32 * i + 8 * g]);
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int t = 0; t < 2; ++t) {
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[i], qw[u][i], acc, 0, 0, 0);
+          for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][i], qw[u][i], acc, 0, 0, 0);
           s[u][t] = acc;
         }
-      }
       // s[u][t][j] is key key_base + 8 g + 4 t + j of column c
       const bool full = key_base + 31 <= full_hi && key_base >= full_lo;  // no masks needed (uniform over the workgroup)
       bf16x8 pf[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      auto soften = [&](int u) {
         float mx = -INFINITY;
         if (full) {
 #pragma unroll
@@ -657,33 +667,52 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
             for (int j = 0; j < 4; ++j) o[u][dt][j] *= alpha;
         }
         lsum[u] += psum;
-      }
+      };
+      auto weigh = [&](int u) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
-#pragma unroll
-        for (int u = 0; u < 2; ++u) o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
-      }
+        for (int dt = 0; dt < DT; ++dt) {
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
+          o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
+        }
+      };
+      soften(0);
+      weigh(0);
+      soften(1);
+      weigh(1);
     };
 
+    // Before round it: block kb0 + it lies in LDS buffer it & 1, block kb0 + it + 1 is on its way into register set
+    // (it + 1) & 1, and the page ids of block kb0 + it + 2 are on their way into page set it & 1.
     if (kb0 < kb1) {
-      fetch_pages(kb0);
-      fetch(kb0);
-      if (kb0 + 1 < kb1) fetch_pages(kb0 + 1);
-      put(0);
+      fetch_pages(kps[0], vps[0], kb0);
+      if (kb0 + 1 < kb1) fetch_pages(kps[1], vps[1], kb0 + 1);
+      fetch(kst[0], vst[0], kps[0], vps[0], kb0);
+      if (kb0 + 1 < kb1) {
+        if (kb0 + 2 < kb1) fetch_pages(kps[0], vps[0], kb0 + 2);  // set 0 is free once block kb0's loads are issued
+        fetch(kst[1], vst[1], kps[1], vps[1], kb0 + 1);
+      }
+      put(kst[0], vst[0], 0);
     }
     __syncthreads();
-    for (int it = 0; it < steps; ++it) {  // both sets pass every barrier; the second may have no block in the last round
+    // One round: the page ids of block it + 3 and then the keys and values of block it + 2 are asked for, this block is
+    // used, and the next block goes from its registers (loaded a round ago) into the other LDS buffer.  Both sets pass
+    // every barrier; the second may have no block in the last round.
+    auto round = [&](bf16x8(&kr_far)[PER_THREAD], bf16x8(&vr_far)[PER_THREAD], int(&kp_far)[PER_THREAD], int(&vp_far)[PER_THREAD],
+                     const bf16x8(&kr_next)[PER_THREAD], const bf16x8(&vr_next)[PER_THREAD], int(&kp_next)[PER_THREAD],
+                     int(&vp_next)[PER_THREAD], int it) {
       const int kb = kb0 + it;
       const int buf = it & 1;
-      const bool more = kb + 1 < kb1;
-      if (more) {
-        fetch(kb + 1);
-        if (kb + 2 < kb1) fetch_pages(kb + 2);
+      if (kb + 2 < kb1) {
+        if (kb + 3 < kb1) fetch_pages(kp_next, vp_next, kb + 3);  // the set that block it + 1's loads were issued from
+        fetch(kr_far, vr_far, kp_far, vp_far, kb + 2);
       }
       if (head_ok && kb < kb1) block(buf, kb);
-      if (more) put(buf ^ 1);
+      if (kb + 1 < kb1) put(kr_next, vr_next, buf ^ 1);
       __syncthreads();
+    };
+    for (int it = 0; it < steps; it += 2) {
+      round(kst[0], vst[0], kps[0], vps[0], kst[1], vst[1], kps[1], vps[1], it);
+      if (it + 1 < steps) round(kst[1], vst[1], kps[1], vps[1], kst[0], vst[0], kps[0], vps[0], it + 1);
     }
 
     // The second set hands its sums to the first, lane by lane (both hold the same columns and channels):
