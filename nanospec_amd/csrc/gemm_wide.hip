@@ -14,7 +14,11 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-#define WIDE_XPAD 8                  // elements of padding per row of the x tile in LDS
+// The x tile in LDS: a row holds its sixteen 8-element pieces in the order 4 i + g for piece 4 g + i (the piece that lane
+// group g needs in its i-th matrix instruction), and rows are 32 bytes longer than their data.  A 16-byte LDS read is
+// served for lanes 0-7 and 16-23 together, i.e. for eight rows at the columns of g and g + 1: this way those sixteen
+// pieces lie in sixteen different groups of four banks.
+#define WIDE_XPAD 16                 // elements of padding per row of the x tile in LDS
 #define WIDE_XROW (128 + WIDE_XPAD)  // elements per row
 
 // partial[(a * ksplit + s) * M * N + m * N + n]: sum over k range s of matrix a (0: w, 1: w2)
@@ -55,6 +59,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
   // The x tile of one k tile: MT*16 rows of 128 k = MT*16*16 pieces of 8; 256 threads take MT pieces each: thread t
   // takes piece t % 16 of rows t / 16 + 16 j, so 16 consecutive threads read one row's 256 contiguous bytes.
   const int xrow0 = tid >> 4, xcol = (tid & 15) * 8;
+  const int xslot = (4 * (tid & 3) + ((tid & 15) >> 2)) * 8;  // where piece tid % 16 = 4 g + i of a row goes in LDS
   // A stage holds what one k tile needs from memory: this wave's fragments of w (and w2) and this thread's pieces of x.
   // DEPTH stages are in flight: the loads of k tile t + DEPTH - 1 are issued before the arithmetic of k tile t.
   constexpr int DEPTH = NACC * NT >= 4 ? 2 : 3;
@@ -85,13 +90,13 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
     // wave that writes buffer b for tile t + 2 has passed the barrier of tile t + 1, which every wave reaches only
     // after it has finished reading b for tile t.
 #pragma unroll
-    for (int j = 0; j < MT; ++j) *reinterpret_cast<bf16x8*>(&xs[buf][xrow0 + 16 * j][xcol]) = sg.xr[j];
+    for (int j = 0; j < MT; ++j) *reinterpret_cast<bf16x8*>(&xs[buf][xrow0 + 16 * j][xslot]) = sg.xr[j];
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][mt * 16 + r][g * 32 + i * 8]);
+        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][mt * 16 + r][(4 * i + g) * 8]);
 #pragma unroll
         for (int a = 0; a < NACC; ++a)
 #pragma unroll
