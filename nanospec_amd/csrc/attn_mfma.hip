@@ -437,6 +437,18 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
 // into sixteen different groups of four banks (the bank-conflict counter reads zero; with 16 bytes of padding every read
 // took twice as long).
 // ------------------------------------------------------------------------------------------------
+// The largest of a value over lanes l, l ^ 16, l ^ 32 and l ^ 48, in all four of them, by the lane-swap instructions of
+// gfx950: swap(a, b) exchanges the upper half of a with the lower half of b (32 lanes), or the odd 16-lane rows of a with
+// the even rows of b; with a = b = x the two results hold a lane's own value and its partner's.  No LDS round trip.
+__device__ __forceinline__ float max_over_lane_rows(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const float m = fmaxf(__uint_as_float(h[0]), __uint_as_float(h[1]));
+  const unsigned v = __float_as_uint(m);
+  const auto q = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
 constexpr bool SHARED_OK = WIDE && PS >= 8 && HD <= 128;  // larger heads do not fit two waves' registers per SIMD
 constexpr int KROW = HD + 16;               // elements of a key's row in LDS
 constexpr int VROW = 32 + 16;               // elements of a channel's row in LDS
@@ -641,8 +653,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
               mx = fmaxf(mx, v);
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = max_over_lane_rows(mx);
         // m[u] is the running maximum of the raw scores (the scale is positive); p = 2^((s - m) scale log2 e)
         const float m_new = fmaxf(m[u], mx);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
