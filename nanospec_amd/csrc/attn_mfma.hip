@@ -463,10 +463,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     constexpr int K_BYTES = 32 * KROW * 2, V_BYTES = HD * VROW * 2, SET_BYTES = 2 * (K_BYTES + V_BYTES);
     constexpr int JOIN_BYTES = 256 * (2 * DT * 4 + 4) * 4;  // what the second set hands to the first: sums, maxima, totals
     __shared__ __align__(16) char smem[2 * SET_BYTES > JOIN_BYTES ? 2 * SET_BYTES : JOIN_BYTES];
-    const int half = threadIdx.x >> 8;  // which set of four waves, i.e. which half of the tile's blocks
+    // What is the same in all lanes of a wave is said to be so (readfirstlane): the loop's branches and the address
+    // arithmetic that depends on the block alone then run on the scalar unit, and no branch is taken under a lane mask.
+    const int half = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);  // which set of four waves, i.e. which half of the tile's blocks
     bf16_t(*lk)[32 * KROW] = reinterpret_cast<bf16_t(*)[32 * KROW]>(smem + half * SET_BYTES);
     bf16_t(*lv)[HD * VROW] = reinterpret_cast<bf16_t(*)[HD * VROW]>(smem + half * SET_BYTES + 2 * K_BYTES);
-    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, g = lane >> 4;
     const int G = a.heads / a.kv_heads;
     const int hblks = (G + 3) / 4;
@@ -479,8 +481,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     const bool head_ok = hin < G;  // a wave without a head still fetches its share of the keys and values
     const int head = kvh * G + (head_ok ? hin : 0);
     const int4 info = *reinterpret_cast<const int4*>(a.tiles + (size_t)tile * TILE_INTS);
-    const int b = info.x, t0 = info.y, q0 = info.z, n = info.w;
-    const int kv_len = a.tiles[(size_t)tile * TILE_INTS + 4];
+    const int b = __builtin_amdgcn_readfirstlane(info.x), t0 = __builtin_amdgcn_readfirstlane(info.y);
+    const int q0 = __builtin_amdgcn_readfirstlane(info.z), n = __builtin_amdgcn_readfirstlane(info.w);
+    const int kv_len = __builtin_amdgcn_readfirstlane(a.tiles[(size_t)tile * TILE_INTS + 4]);
     const int* table = a.block_table + (size_t)b * a.table_stride;
     constexpr int psh = __builtin_ctz(PS), pmask = PS - 1;
 
@@ -571,19 +574,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     bf16x8 kst[2][PER_THREAD], vst[2][PER_THREAD];
     // Otherwise addresses are kept inside held pages: a key outside [wlo, whi) is masked anyway.
     auto fetch_pages = [&](int(&kp)[PER_THREAD], int(&vp)[PER_THREAD], int kb) {
-      if (inside(kb)) {
-        const int* row = table + kb * PPB;
+      const bool in = inside(kb);
 #pragma unroll
-        for (int r = 0; r < PER_THREAD; ++r) {
-          kp[r] = row[k_slot[r]];
-          vp[r] = row[v_slot[r]];
-        }
-      } else {
-#pragma unroll
-        for (int r = 0; r < PER_THREAD; ++r) {
-          kp[r] = table[min(max(kb * 32 + k_key[r], wlo), whi - 1) >> psh];
-          vp[r] = table[min(max(kb * 32 + v_kq[r] * 8, vlo), vhi) >> psh];
-        }
+      for (int r = 0; r < PER_THREAD; ++r) {  // one load each, from an index chosen beforehand
+        const int ks = in ? kb * PPB + k_slot[r] : min(max(kb * 32 + k_key[r], wlo), whi - 1) >> psh;
+        const int vs = in ? kb * PPB + v_slot[r] : min(max(kb * 32 + v_kq[r] * 8, vlo), vhi) >> psh;
+        kp[r] = table[ks];
+        vp[r] = table[vs];
       }
     };
     auto fetch = [&](bf16x8(&kr)[PER_THREAD], bf16x8(&vr)[PER_THREAD], const int(&kp)[PER_THREAD], const int(&vp)[PER_THREAD], int kb) {
