@@ -96,7 +96,8 @@ struct KVBlock {
 // 8B shape).  The kernel chooses by the number of keys over all layers, which the host leaves in the tiles.
 template <int QT, bool PREFETCH, bool COOP, bool NT>
 __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // what is the same in all lanes of a wave is said to be so (readfirstlane): branches on it are then scalar ones
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int G = a.heads / a.kv_heads;
   const int hblks = (G + a.hp - 1) / a.hp;
@@ -139,6 +140,8 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
     kb0 = kb0 + split * per;
     kb1 = min(kb1, kb0 + per);
   }
+  kb0 = __builtin_amdgcn_readfirstlane(kb0);
+  kb1 = __builtin_amdgcn_readfirstlane(kb1);
 
   // Q^T fragments of this lane's columns
   bf16x8 qw[QT][WIDE ? NQ : 1];
@@ -179,18 +182,26 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
 
   // The page ids of up to 64 consecutive pages are held one per lane and handed round by lane exchange, so that the
   // chain of loads of a block is one load long (keys and values) rather than two (block table, then keys and values).
+  // The ids of the 64 pages after those are asked for at the same time and taken over when a block reaches them: the
+  // lane exchange then never reads a register that a load may still be writing, so nothing waits for the loads in
+  // flight (a wait for the page ids would be a wait for all the keys and values asked for before them).
   const int last_page = max(whi - 1, 0) >> psh;
-  int page_base = 0x40000000, my_page = 0;
+  int page_base = __builtin_amdgcn_readfirstlane((kb0 * 32) >> psh);
+  int my_page = table[min(page_base + lane, last_page)];
+  int next_pages = table[min(page_base + 64 + lane, last_page)];
+  asm volatile("" : "+v"(my_page));  // here, once, the first ids are waited for (on every path into the loops below)
   auto page_of = [&](int key) { return __shfl(my_page, (key >> psh) - page_base, 64); };
 
   // Issue the loads of block kb: keys, values.  Addresses are kept inside held pages: a key outside [wlo, whi) is masked
   // anyway.
+  // A wave's blocks come in rising order, the first one's first page is page_base, and a block's pages never straddle
+  // a multiple of 64 pages from there (32 keys are a power of two of pages, or a part of one page).
   auto pages_for = [&](int kb) {
-    const int key_base = kb * 32;
-    const int p_lo = key_base >> psh, p_hi = (key_base + 31) >> psh;
-    if (p_lo < page_base || p_hi >= page_base + 64) {  // uniform over the wave
-      page_base = p_lo;
-      my_page = table[min(page_base + lane, last_page)];
+    const int p_hi = (kb * 32 + 31) >> psh;
+    while (p_hi >= page_base + 64) {  // uniform over the wave; once in 64 pages
+      page_base += 64;
+      my_page = next_pages;
+      next_pages = table[min(page_base + 64 + lane, last_page)];
     }
   };
   auto load_k = [&](KVBlock& blk, int kb) {
