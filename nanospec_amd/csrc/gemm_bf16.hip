@@ -69,21 +69,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
   constexpr int NACC = EPI == EPI_SILU_MUL ? 2 : 1;
   __shared__ float red[WAVES][NACC * MT][256];
   __shared__ float rinv_s[MT * 16];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in a wave's lanes
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int KT = (K + 127) / 128;
   // What the epilogue needs besides the sums is asked for now and used after the weights have streamed.
   // Consumer: wave v takes rows v, v + WAVES, ...; its lanes take the producer's workgroups in turn.
   constexpr int RPW = (16 + WAVES - 1) / WAVES, PRE = 4;
+  // The loads are unconditional, from indices kept inside the arrays, and what lies outside is dropped where the values
+  // are used: a load under a condition would be waited for on the spot, before the weights' loads have even started.
   float ssq_pre[RPW][PRE];
   if (nl.ssq_in) {
 #pragma unroll
     for (int rr = 0; rr < RPW; ++rr)
 #pragma unroll
       for (int i = 0; i < PRE; ++i) {
-        const int m = wave + rr * WAVES, p = lane + 64 * i;
-        ssq_pre[rr][i] = (m < M && p < nl.parts_in) ? nl.ssq_in[(size_t)m * nl.parts_in + p] : 0.f;
+        const int m = min(wave + rr * WAVES, M - 1), p = min(lane + 64 * i, nl.parts_in - 1);
+        ssq_pre[rr][i] = nl.ssq_in[(size_t)m * nl.parts_in + p];
       }
   }
   // Producer: thread e <-> (column n0 + e / 16, row e % 16), one or two elements per thread.
@@ -92,11 +94,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
   if (EPI == EPI_RESID_NORM) {
 #pragma unroll
     for (int i = 0; i < EPT; ++i) {
-      const int e = threadIdx.x + i * WAVES * 64;
-      const int n = n0 + (e >> 4), m = e & 15;
-      const bool ok = e < 256 && n < N && m < M;
-      resid_pre[i] = ok ? (float)nl.resid[(size_t)m * nl.resid_stride + n] : 0.f;
-      wnext_pre[i] = ok ? (float)nl.w_next[n] : 0.f;
+      const int e = min(threadIdx.x + i * WAVES * 64, 255);
+      const int n = min(n0 + (e >> 4), N - 1), m = min(e & 15, M - 1);
+      resid_pre[i] = (float)nl.resid[(size_t)m * nl.resid_stride + n];
+      wnext_pre[i] = (float)nl.w_next[n];
     }
   }
   const bf16_t* wbase = wt + (size_t)blockIdx.x * KT * 2048 + lane * 8;
@@ -173,7 +174,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
       const int m = wave + rr * WAVES;
       float v = 0.f;
 #pragma unroll
-      for (int i = 0; i < PRE; ++i) v += ssq_pre[rr][i];
+      for (int i = 0; i < PRE; ++i) {
+        asm volatile("" : "+v"(ssq_pre[rr][i]));  // first used here, after the loop: no arithmetic on it may move up to its load
+        v += (m < M && lane + 64 * i < nl.parts_in) ? ssq_pre[rr][i] : 0.f;
+      }
       if (m < M)
         for (int p = lane + 64 * PRE; p < nl.parts_in; p += 64) v += nl.ssq_in[(size_t)m * nl.parts_in + p];
 #pragma unroll
@@ -253,6 +257,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
       const int le = (((nl_ >> 2) * 16 + m) << 2) + (nl_ & 3);  // where the product's sums for (row, column) sit
       const int n = n0 + nl_;
       float q = 0.f;
+      asm volatile("" : "+v"(resid_pre[i]), "+v"(wnext_pre[i]));  // first used here (see the sums of squares above)
       if (n < N && m < M) {
         float s = 0.f;
 #pragma unroll
