@@ -79,18 +79,22 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
       }
     }
 #pragma unroll
+    // No load stands under a condition (the compiler would wait for it on the spot, and with it for every load in
+    // flight): rows beyond M repeat row M - 1, whose sums are never stored, and a piece beyond K is read from inside
+    // the row and replaced by zeros when it goes into LDS.
     for (int j = 0; j < MT; ++j) {
-      const int m = xrow0 + 16 * j;
-      const int k = kt * 128 + xcol;
-      sg.xr[j] = (m < M && k < K) ? *reinterpret_cast<const bf16x8*>(x + (size_t)m * x_stride + k) : zero;
+      const int m = min(xrow0 + 16 * j, M - 1);
+      const int k = min(kt * 128 + xcol, K - 8);
+      sg.xr[j] = *reinterpret_cast<const bf16x8*>(x + (size_t)m * x_stride + k);
     }
   };
-  auto step = [&](const Stage& sg, int buf) {
+  auto step = [&](const Stage& sg, int buf, int kt) {
+    const bool in_k = kt * 128 + xcol < K;
     // x pieces into LDS, then every wave multiplies its w fragments with the whole tile.  One barrier per k tile: a
     // wave that writes buffer b for tile t + 2 has passed the barrier of tile t + 1, which every wave reaches only
     // after it has finished reading b for tile t.
 #pragma unroll
-    for (int j = 0; j < MT; ++j) *reinterpret_cast<bf16x8*>(&xs[buf][xrow0 + 16 * j][xslot]) = sg.xr[j];
+    for (int j = 0; j < MT; ++j) *reinterpret_cast<bf16x8*>(&xs[buf][xrow0 + 16 * j][xslot]) = in_k ? sg.xr[j] : zero;
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -108,13 +112,23 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
 #pragma unroll
   for (int d = 0; d < DEPTH - 1; ++d)
     if (kt0 + d < kt1) fetch(st[d], kt0 + d);
-  for (int kt = kt0; kt < kt1; kt += DEPTH) {
+  // In the body of the first loop every load is unconditional, so the compiler's count of what may stay in flight is
+  // exact there; the last tiles (fewer than two rounds of DEPTH) run with the checks.
+  int kt = kt0;
+  for (; kt + 2 * DEPTH - 2 < kt1; kt += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      fetch(st[(d + DEPTH - 1) % DEPTH], kt + d + DEPTH - 1);
+      step(st[d], (kt + d - kt0) & 1, kt + d);
+    }
+  }
+  for (; kt < kt1; kt += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const int cur = kt + d;
       if (cur < kt1) {
         if (cur + DEPTH - 1 < kt1) fetch(st[(d + DEPTH - 1) % DEPTH], cur + DEPTH - 1);
-        step(st[d], (cur - kt0) & 1);
+        step(st[d], (cur - kt0) & 1, cur);
       }
     }
   }
