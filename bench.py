@@ -20,10 +20,15 @@ import time
 HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-SHAPE_8B = dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+SHAPES = {}
+SHAPES["8b"] = SHAPE_8B = dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
                 num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=131072,
                 rope_scaling=dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192),
                 tie_word_embeddings=False)
+SHAPES["1b"] = dict(SHAPE_8B, hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, head_dim=64, tie_word_embeddings=True,
+                    rope_scaling=dict(SHAPE_8B["rope_scaling"], factor=32.0))
+SHAPES["70b"] = dict(SHAPE_8B, hidden_size=8192, intermediate_size=28672, num_hidden_layers=80, num_attention_heads=64)
+SHAPE_NAMES = {"8b": "Llama-3.1-8B shape", "1b": "Llama-3.2-1B shape", "70b": "Llama-3.1-70B shape"}
 
 
 def weight_bytes(c, esize: int) -> int:
@@ -117,6 +122,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true")
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (--gpus must be 1)")
@@ -127,7 +133,7 @@ def main() -> int:
     from nanospec_amd import LlamaConfig
     from nanospec_amd.loader import random_model
 
-    shape = dict(SHAPE_8B)
+    shape = dict(SHAPES[a.shape])
     full_layers = shape["num_hidden_layers"]
     if a.layers:
         shape["num_hidden_layers"] = a.layers
@@ -159,11 +165,11 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * k / d, 1)
 
     line = {
-        "metric": "decode tok/s at bs 8, ctx 2048->4096 (Llama-3.1-8B shape, bf16); prefill tok/s @2048 tok",
+        "metric": f"decode tok/s at bs {a.batch}, ctx 2048->4096 ({SHAPE_NAMES[a.shape]}, {a.dtype}); prefill tok/s @2048 tok",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
-        "config": {"model": "Llama-3.1-8B shape", "layers": shape["num_hidden_layers"], "layers_of_shape": full_layers,
+        "config": {"model": SHAPE_NAMES[a.shape], "layers": shape["num_hidden_layers"], "layers_of_shape": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": prompt, "ctx_first_step": round(ctx0, 1),
