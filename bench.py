@@ -61,7 +61,8 @@ def decode_run(model, cfg, batch: int, prompt_len: int, first_ctx: int, steps: i
     # few tokens ahead of the last when the clock starts.  No request ends before the clock stops: the engine enqueues
     # each step one ahead of the one it waits for, so the step enqueued in the last warm-up call has run before the
     # clock starts and the last timed call enqueues one more, and the clock covers the GPU's work of exactly ``steps`` steps.
-    ahead = batch * -(-first_ctx // 2048) + 2
+    # (a prompt takes one step per 2,048 tokens, and one more when the decode rows of the step leave it less than that)
+    ahead = batch * (-(-first_ctx // 2048) + 1) + 2
     total = first_ctx + ahead + warmup + steps + 2
     blocks = batch * -(-(total + 1) // block_size) + 2
     eng = Engine(model, EngineConfig(num_blocks=blocks, block_size=block_size, max_admit=batch, max_running=batch,

@@ -1,4 +1,5 @@
-// bfloat16 matrix products on the matrix cores for 17 to 64 rows (decode at large batch, short portions):
+// bfloat16 matrix products on the matrix cores for 17 to 64 rows, and for up to 128 rows of one matrix with one row tile
+// per wave (decode at large batch, short portions):
 //   out[M, N] = x[M, K] . w[N, K]^T,  32-bit accumulation, weights in the tiled layout of gemm_bf16.hip.
 //
 // With this many rows the traffic of x counts: a workgroup of 4 waves owns 64 rows of w (16 per wave) and all its
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
   const int xslot = (4 * (tid & 3) + ((tid & 15) >> 2)) * 8;  // where piece tid % 16 = 4 g + i of a row goes in LDS
   // A stage holds what one k tile needs from memory: this wave's fragments of w (and w2) and this thread's pieces of x.
   // DEPTH stages are in flight: the loads of k tile t + DEPTH - 1 are issued before the arithmetic of k tile t.
-  constexpr int DEPTH = NACC * NT >= 4 ? 2 : 3;
+  constexpr int DEPTH = (NACC * NT >= 4 || MT > 6) ? 2 : 3;  // what the registers hold at two waves per SIMD
   struct Stage {
     bf16x8 wf[NACC][NT][4];
     bf16x8 xr[MT];
@@ -208,13 +209,24 @@ static int launch_wide(float* partial, const bf16_t* x, const bf16_t* wt, const 
   return ns_launch_status();
 }
 
+// 65 to 128 rows: one matrix, one row tile per wave (the x tile takes 72 KiB of LDS at 128 rows).
+template <int MT>
+static int launch_wide_tall(float* partial, const bf16_t* x, const bf16_t* wt, int M, int N, int K, int x_stride, int ksplit,
+                            void* direct_out, int out_stride, int out_f32, hipStream_t stream) {
+  const int row_tiles = (N + 15) / 16;
+  dim3 grid((row_tiles + 3) / 4, ksplit);
+  gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
+  return ns_launch_status();
+}
+
 // workspace: (wt2 ? 2 : 1) * ksplit * M * N floats (unused with ksplit == 1).  epi 0: store; 1: silu(x.w^T) * (x.w2^T).
 // defer (with ksplit > 1 and epi 0): the ranges stay in the workspace as [ksplit][M][N] and nothing is written to out; they
 // are added later by ns_wide_reduce or by a norm that reads them (ns_rmsnorm_partial).
 extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
                                  int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer,
                                  hipStream_t stream) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
+  if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
+  if (M > 64 && (wt2 != nullptr || nt != 1)) return NS_ERR_BAD_ARG;  // 65 to 128 rows: one matrix, one row tile per wave
   if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
   const int KT = (K + 127) / 128;
   if (ksplit < 1 || ksplit > KT || ksplit > 65535 || (nt != 1 && nt != 2) || (ksplit > 1 && !workspace)) return NS_ERR_BAD_ARG;
@@ -226,7 +238,11 @@ extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, cons
     case 1: st = launch_wide<1>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
     case 2: st = launch_wide<2>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
     case 3: st = launch_wide<3>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
-    default: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
+    case 4: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, direct, out_stride, out_f32, stream); break;
+    case 5: st = launch_wide_tall<5>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
+    case 6: st = launch_wide_tall<6>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
+    case 7: st = launch_wide_tall<7>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
+    default: st = launch_wide_tall<8>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
   }
   if (st != NS_OK || direct) return st;
   if (defer) return epi == 0 ? NS_OK : NS_ERR_BAD_ARG;

@@ -230,6 +230,7 @@ def linear_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = 
 
 
 SKINNY_MAX_ROWS = 64
+WIDE_TALL_ROWS = 128  # ``linear_wide`` with one matrix and one row tile per wave takes this many rows
 
 
 class TiledWeight:
@@ -264,8 +265,8 @@ class TiledWeight:
         return out
 
 
-def tiled_takes(x: torch.Tensor, k: int) -> bool:
-    return (x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and k % 8 == 0 and x.stride(0) % 8 == 0
+def tiled_takes(x: torch.Tensor, k: int, max_rows: int = SKINNY_MAX_ROWS) -> bool:
+    return (x.dtype == torch.bfloat16 and x.shape[0] <= max_rows and k % 8 == 0 and x.stride(0) % 8 == 0
             and x.stride(1) == 1 and x.data_ptr() % 16 == 0)
 
 
@@ -352,10 +353,11 @@ def linear_resid_norm(x: torch.Tensor, w: TiledWeight, resid: torch.Tensor, next
     return PreNormed(x_next, ssq, w.n, eps)
 
 
-def wide_plan(n: int, k: int) -> tuple[int, int]:
-    """(ranges K is cut into, 16-row tiles per wave) of ``linear_wide``: two tiles per wave when there are rows enough,
+def wide_plan(n: int, k: int, rows: int = SKINNY_MAX_ROWS) -> tuple[int, int]:
+    """(ranges K is cut into, 16-row tiles per wave) of ``linear_wide``: two tiles per wave when there are rows enough
+    (and at most 64 rows of x),
     then enough ranges that the workgroups fill the GPU, with at least four k tiles of 128 per range."""
-    nt = 2 if n >= 8192 else 1
+    nt = 2 if n >= 8192 and rows <= SKINNY_MAX_ROWS else 1
     row_groups = -(-n // (64 * nt))
     k_tiles = -(-k // 128)
     return max(1, min(16, k_tiles // 4, round(640 / row_groups))), nt
@@ -363,18 +365,21 @@ def wide_plan(n: int, k: int) -> tuple[int, int]:
 
 def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
                 out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0, defer: bool = False):
-    """bfloat16 x @ w.T for up to 64 rows from a tiled weight, with the tile of x shared through LDS by the four waves of
+    """bfloat16 x @ w.T for up to 64 rows from a tiled weight (up to 128 with ``nt=1`` and no ``w2``), with the tile of x
+    shared through LDS by the four waves of
     a workgroup and K cut into ``ksplit`` ranges that a second kernel adds up; with ``w2``: silu(x @ w.T) * (x @ w2.T).
     ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values (none for a single range).  ``defer`` (not with
     ``w2``): with more than one range the second kernel is left out and a ``PartialSums`` over the workspace comes back."""
     _gpu(x, out, workspace)
-    if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k):
-        raise KernelRefused(f"linear_wide takes bfloat16 x [rows <= {SKINNY_MAX_ROWS}, {w.k}] with an inner size that is a "
+    if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k, WIDE_TALL_ROWS):
+        raise KernelRefused(f"linear_wide takes bfloat16 x [rows <= {WIDE_TALL_ROWS}, {w.k}] with an inner size that is a "
                             f"multiple of 8; got {tuple(x.shape)} {x.dtype}")
     m = x.shape[0]
     want = torch.float32 if out_f32 else x.dtype
-    plan = wide_plan(w.n, w.k)
+    plan = wide_plan(w.n, w.k, m)
     ksplit, nt = ksplit or plan[0], nt or plan[1]
+    if m > SKINNY_MAX_ROWS and (w2 is not None or nt != 1):
+        raise KernelRefused(f"linear_wide takes more than {SKINNY_MAX_ROWS} rows only for one matrix with one row tile per wave")
     defer = defer and ksplit > 1 and w2 is None and not out_f32
     if out is None and not defer:
         out = torch.empty((m, w.n), dtype=want, device=x.device)

@@ -6,7 +6,8 @@ matrix-core mode of reduced precision is ever used).
 bfloat16: decode and short portions (up to ``STREAM_ROWS`` rows) run the hand-written matrix-core kernel that streams
 the weights once; it reads them in a layout re-laid at load time (``kernels.ops.TiledWeight``) in which every load
 of a wave is one contiguous kilobyte.  17 to 64 rows run a second hand-written kernel on the same layout (x shared
-through LDS, K cut into ranges) where it is ahead of the library.  More rows go to the platform's GEMM library on the
+through LDS, K cut into ranges) where it is ahead of the library, and so do products of up to 128 rows that end in the
+residual stream (at 65 to 128 rows the library takes two to three times as long for them).  More rows go to the platform's GEMM library on the
 plain layout, as the reference's nn.Linear does (model/llama.py:168-171).  32-bit results (logits) always come from the
 hand-written kernels, in slices of 64 rows, so that no logit is rounded to bfloat16.  Both layouts are kept in memory unless
 ``keep_plain=False``.
@@ -38,8 +39,8 @@ class IntoResidual:
       * ``kernels.ops.PreNormed``: ``resid += output`` has been done in place and the norm needs no kernel of its own
         (at most 16 rows: the product's epilogue did the sum and the norm's statistics);
       * ``kernels.ops.PartialSums``: the ranges of a product whose K was cut, which the norm kernel adds up as it reads
-        them (17 to 64 rows);
-      * ``kernels.ops.Added``: ``resid += output`` has been done in place by the product itself (more than 64 rows, through
+        them (17 to 128 rows);
+      * ``kernels.ops.Added``: ``resid += output`` has been done in place by the product itself (more rows, through
         the library), the norm still has its kernel;
       * a tensor: the output, still to be added by the norm kernel.
     ``next_weight``, ``eps``: that norm's weight and epsilon.  ``x_next`` (like resid), ``ssq`` (float32 [rows,
@@ -77,9 +78,9 @@ class LinearWeight:
             x_next = link.x_next if link.x_next is not None else take(tuple(link.resid.shape), link.resid.dtype)
             ssq = link.ssq if link.ssq is not None else take((m, -(-self.n // 16)), torch.float32)
             return ops.linear_resid_norm(x, self.tiled, link.resid, link.next_weight, link.eps, x_next=x_next, ssq=ssq)
-        if (self.tiled is not None and STREAM_ROWS < m <= ops.SKINNY_MAX_ROWS and (self.plain is None or self.n <= WIDE_MAX_N)
+        if (self.tiled is not None and STREAM_ROWS < m <= ops.WIDE_TALL_ROWS and (self.plain is None or self.n <= WIDE_MAX_N)
                 and x.dtype == torch.bfloat16 and ops.tiled_takes(x[:1], self.k)):
-            ksplit, nt = ops.wide_plan(self.n, self.k)
+            ksplit, nt = ops.wide_plan(self.n, self.k, m)
             need = ksplit * m * self.n
             ws = None
             if ksplit > 1 and link.carry is not None and link.carry.numel() >= need:

@@ -93,7 +93,7 @@ class DecoderModel:
         order = self.spec.run_order
         # buffers for what one block hands to the next (see PreNormBlock.forward)
         sums = ctx.arena.take((n, -(-self.spec.hidden // 16)), torch.float32)
-        carry = ctx.arena.take((16 * n * self.spec.hidden,), torch.float32) if 16 < n <= ops.SKINNY_MAX_ROWS and self.dtype == torch.bfloat16 else None
+        carry = ctx.arena.take((16 * n * self.spec.hidden,), torch.float32) if 16 < n <= ops.WIDE_TALL_ROWS and self.dtype == torch.bfloat16 else None
         for i, call in enumerate(order):
             layer = self.layers[call.layer]
             if getattr(layer, "links_blocks", False) and i + 1 < len(order):

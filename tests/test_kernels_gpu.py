@@ -287,7 +287,33 @@ def test_product_that_updates_the_residual_and_feeds_the_next_norm(m, hidden, in
     assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * up).max() <= 2.0
 
 
-@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("m", [65, 81, 100, 113, 128])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (4096, 2056)])
+def test_linear_wide_up_to_128_rows(m, n, k):
+    """65 to 128 rows: one matrix, one row tile per wave; every count of ranges, sizes off the tile; other forms refused."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m + 3, k + 8, dtype=torch.bfloat16, device=DEV)[:m, :k]
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    wt = ops.TiledWeight(w)
+    ref = x.cpu().float() @ w.cpu().float().T
+    k_tiles = -(-k // 128)
+    for ks in sorted({1, min(2, k_tiles), min(5, k_tiles), k_tiles, 0}):
+        out = ops.linear_wide(x, wt, out_f32=True, ksplit=ks, nt=0 if ks == 0 else 1)
+        torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
+    assert ulps_of_row_max(ops.linear_wide(x, wt).cpu(), ref).max() <= 1.0
+    if k_tiles >= 2:
+        part = ops.linear_wide(x, wt, ksplit=2, nt=1, defer=True)
+        assert torch.equal(ops.reduce_partial(part), ops.linear_wide(x, wt, ksplit=2, nt=1))
+    with pytest.raises(ops.KernelRefused):
+        ops.linear_wide(x, wt, nt=2)
+    with pytest.raises(ops.KernelRefused):
+        ops.linear_wide(x, wt, w2=wt)
+    with pytest.raises(ops.KernelRefused):
+        ops.linear_wide(torch.randn(129, k, dtype=torch.bfloat16, device=DEV), wt)
+
+
+@pytest.mark.parametrize("m", [17, 40, 64, 97, 128])
 @pytest.mark.parametrize("hidden,inner,ksplit", [(136, 1024, 4), (4096, 1024, 2), (72, 512, 3)])
 def test_ranges_of_a_product_added_by_the_norm_that_reads_them(m, hidden, inner, ksplit):
     """The 17-to-64-row product leaves the ranges of K unadded; the RMS norm adds them as it reads them, with the residual
