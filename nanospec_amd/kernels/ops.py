@@ -314,8 +314,8 @@ def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight 
         raise KernelRefused("linear_tiled: out has the wrong shape or dtype")
     if w2 is not None and (w2.n != w.n or w2.k != w.k):
         raise KernelRefused("linear_tiled: w2 must match w")
-    if waves == 0:
-        waves = 8 if w.k >= 8192 or (w.n // 16 < 512 and w.k >= 2048) else 4
+    if waves == 0:  # with more than 8 rows eight waves were never behind four at the shapes measured
+        waves = 8 if w.k >= 8192 or ((w.n // 16 < 512 or m > 8) and w.k >= 2048) else 4
     _check(build.core().ns_gemm_tiled_bf16(_ptr(out), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None), c_int(m),
                                            c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
                                            c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(waves),

@@ -29,6 +29,7 @@ class Layouts:
 
 
 STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured
+WIDE_HEAD_ROWS = 12  # above this many rows a wide 32-bit product (the head) is faster through the 17-to-64-row kernel
 WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
 #                    32-bit results, which the library does not give); wider products go to the library
 
@@ -111,6 +112,8 @@ class LinearWeight:
         if self.dtype == torch.float32 or self.k % 8 or not ops.tiled_takes(x[:1], self.k):
             return ops.linear_generic(x, self.plain, out=out, out_f32=out_f32)
         m = x.shape[0]
+        if self.tiled is not None and WIDE_HEAD_ROWS < m <= STREAM_ROWS and out_f32 and self.n >= 8192:
+            return ops.linear_wide(x, self.tiled, out=out, out_f32=True, ksplit=1, nt=1)
         if self.tiled is not None and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled, out=out, out_f32=out_f32)
         if self.tiled is not None and m <= ops.SKINNY_MAX_ROWS and (out_f32 or self.plain is None or self.n <= WIDE_MAX_N):
