@@ -33,44 +33,53 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
                                                             const float* __restrict__ temperature,
                                                             const int* __restrict__ top_k, const float* __restrict__ top_p,
                                                             const float* __restrict__ uniform, int vocab) {
+  constexpr int WAVES = SP_THREADS / NS_WAVE;
   __shared__ float scratch[16];
-  __shared__ float prefix[SP_THREADS];
+  __shared__ float chunk_sum[WAVES];
+  __shared__ int chunk_last[WAVES];
   __shared__ int s_idx;
   const int r = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (size_t)r * row_stride;
+  const bool wide = (((uintptr_t)z) & 15) == 0;
+  const int n4 = wide ? vocab >> 2 : 0;
+  const float4* z4 = reinterpret_cast<const float4*>(z);
 
-  // arg-max of the raw logits (lowest index among equals) and their log-sum-exp, in one pass: every thread keeps the
-  // sum of exp(z - its own maximum so far)
-  float best = -INFINITY, se = 0.f;
+  // First pass: the arg-max of the raw logits, lowest index among equals (a thread meets its indices in rising order).
+  // Second pass: the sum of exp(z - max).  Two cheap passes instead of one that rescales a running sum at every element:
+  // the row is read by a single compute unit and its arithmetic, not the memory, sets the time.
+  float best = -INFINITY;
   int best_i = 0x7fffffff;
   auto take = [&](float v, int i) {
     if (v > best) {
-      se = se * expf(best - v) + 1.f;  // best = -inf: se is still 0
       best = v;
       best_i = i;
-    } else if (v > -INFINITY) {
-      se += expf(v - best);
     }
   };
-  if ((((uintptr_t)z) & 15) == 0) {
-    const int n4 = vocab >> 2;
-    const float4* z4 = reinterpret_cast<const float4*>(z);
-    for (int i = tid; i < n4; i += SP_THREADS) {
-      const float4 v = z4[i];
-      take(v.x, 4 * i);
-      take(v.y, 4 * i + 1);
-      take(v.z, 4 * i + 2);
-      take(v.w, 4 * i + 3);
-    }
-    for (int i = 4 * n4 + tid; i < vocab; i += SP_THREADS) take(z[i], i);
-  } else {
-    for (int i = tid; i < vocab; i += SP_THREADS) take(z[i], i);
+  for (int i = tid; i < n4; i += SP_THREADS) {
+    const float4 v = z4[i];
+    take(v.x, 4 * i);
+    take(v.y, 4 * i + 1);
+    take(v.z, 4 * i + 2);
+    take(v.w, 4 * i + 3);
   }
+  for (int i = 4 * n4 + tid; i < vocab; i += SP_THREADS) take(z[i], i);
   const float zmax = block_max(best, scratch);
   if (tid == 0) s_idx = 0x7fffffff;
   __syncthreads();
   if (best == zmax) atomicMin(&s_idx, best_i);
-  const float lse = zmax + logf(block_sum(best > -INFINITY ? se * expf(best - zmax) : 0.f, scratch));  // barriers inside publish s_idx
+  float se = 0.f;
+  auto add = [&](float v) {
+    if (v > -INFINITY) se += __expf(v - zmax);  // not for NaN
+  };
+  for (int i = tid; i < n4; i += SP_THREADS) {
+    const float4 v = z4[i];
+    add(v.x);
+    add(v.y);
+    add(v.z);
+    add(v.w);
+  }
+  for (int i = 4 * n4 + tid; i < vocab; i += SP_THREADS) add(z[i]);
+  const float lse = zmax + logf(block_sum(zmax > -INFINITY ? se : 0.f, scratch));  // barriers inside publish s_idx
   const int amax = s_idx < vocab ? s_idx : 0;  // a row without a single comparable value (all NaN or -inf) names token 0
   const float T = temperature[r];
   if (T <= 0.f) {
@@ -108,49 +117,159 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
     cut = ord2f(lo);
   }
 
-  // inverse CDF in vocabulary order: each thread owns a contiguous range
-  const int per = (vocab + SP_THREADS - 1) / SP_THREADS;
-  const int i0 = min(vocab, tid * per), i1 = min(vocab, i0 + per);
+  // Inverse CDF in vocabulary order.  Every wave owns a contiguous chunk (a multiple of 256 tokens) and adds up what
+  // stays of it, its lanes reading neighbouring tokens; then the chunk in which the running sum passes u * total is found.
+  const bool filtered = cut > -INFINITY;
+  const float inv_t = 1.f / T;
+  // what a token weighs and whether it stays; without a cut everything but NaN stays and the weight needs no division
+  auto weigh = [&](float v, bool& kept) -> float {
+    if (filtered) {
+      const float sv = v / T;  // the very expression whose values the cut was found among
+      kept = sv >= cut;
+      return kept ? expf(sv - smax) : 0.f;
+    }
+    kept = v == v;
+    return kept ? __expf((v - zmax) * inv_t) : 0.f;
+  };
+  const int lane = tid & (NS_WAVE - 1), wave = tid / NS_WAVE;
+  const int chunk = (((vocab + WAVES - 1) / WAVES) + 4 * NS_WAVE - 1) & ~(4 * NS_WAVE - 1);
+  const int c0 = min(vocab, wave * chunk), c1 = min(vocab, c0 + chunk);
   float mine = 0.f;
   int last_kept = -1;
-  for (int i = i0; i < i1; ++i) {
-    const float s = z[i] / T;
-    if (s >= cut) { mine += expf(s - smax); last_kept = i; }
+  auto count = [&](float v, int i) {
+    bool kept;
+    mine += weigh(v, kept);
+    if (kept) last_kept = i;
+  };
+  const int c4 = wide ? (c1 - c0) >> 2 : 0;  // 16-byte pieces of the chunk (it starts at a multiple of 256 tokens)
+  for (int q = lane; q < c4; q += NS_WAVE) {
+    const float4 v = z4[(c0 >> 2) + q];
+    const int i = c0 + 4 * q;
+    count(v.x, i);
+    count(v.y, i + 1);
+    count(v.z, i + 2);
+    count(v.w, i + 3);
   }
-  prefix[tid] = mine;
-  __syncthreads();
-  if (tid == 0) {
-    float run = 0.f;
-    for (int i = 0; i < SP_THREADS; ++i) { const float v = prefix[i]; prefix[i] = run; run += v; }
-    scratch[0] = run;
-    s_idx = 0x7fffffff;
+  for (int i = c0 + 4 * c4 + lane; i < c1; i += NS_WAVE) count(z[i], i);
+  mine = wave_sum(mine);
+#pragma unroll
+  for (int o = NS_WAVE / 2; o > 0; o >>= 1) last_kept = max(last_kept, __shfl_xor(last_kept, o, NS_WAVE));
+  if (lane == 0) {
+    chunk_sum[wave] = mine;
+    chunk_last[wave] = last_kept;
   }
   __syncthreads();
-  const float total = scratch[0];
+  float total = 0.f;
+  for (int j = 0; j < WAVES; ++j) total += chunk_sum[j];
   const float target = uniform[r] * total;
-  float run = prefix[tid];
-  for (int i = i0; i < i1; ++i) {
-    const float s = z[i] / T;
-    if (s >= cut) {
-      run += expf(s - smax);
-      if (run > target) { atomicMin(&s_idx, i); break; }
+  int sel = -1, last_all = -1;
+  float before = 0.f, sel_before = 0.f;
+  for (int j = 0; j < WAVES; ++j) {
+    if (sel < 0 && before + chunk_sum[j] > target) {
+      sel = j;
+      sel_before = before;
+    }
+    before += chunk_sum[j];
+    last_all = max(last_all, chunk_last[j]);
+  }
+  // The chunk in which the passing lies is cut once more, into a piece per wave; the piece in which it lies is walked by
+  // its wave alone: the sums of eight runs of 64 tokens at a time (their loads and lane exchanges do not wait for one
+  // another), then a scan over the lanes of the run in which the passing lies.
+  constexpr int AHEAD = 8;
+  const int piece = chunk / WAVES;  // a multiple of 16 tokens
+  const int s_lo = sel < 0 ? 0 : min(vocab, sel * chunk), s_hi = sel < 0 ? 0 : min(vocab, s_lo + chunk);
+  const int p0 = min(s_hi, s_lo + wave * piece), p1 = min(s_hi, p0 + piece);
+  __syncthreads();  // chunk_sum and chunk_last have been read by everyone: they now hold the pieces
+  int tok = -1, owner = -1;
+  if (sel >= 0) {
+    float psum = 0.f;
+    int plast = -1;
+    for (int b0 = p0; b0 < p1; b0 += AHEAD * NS_WAVE) {
+      float v[AHEAD];
+#pragma unroll
+      for (int j = 0; j < AHEAD; ++j) v[j] = z[min(b0 + j * NS_WAVE + lane, p1 - 1)];  // no load under a condition
+#pragma unroll
+      for (int j = 0; j < AHEAD; ++j) {
+        bool kept;
+        const float w = weigh(v[j], kept);
+        if (b0 + j * NS_WAVE + lane < p1) {
+          psum += w;
+          if (kept) plast = b0 + j * NS_WAVE + lane;
+        }
+      }
+    }
+    psum = wave_sum(psum);
+#pragma unroll
+    for (int o = NS_WAVE / 2; o > 0; o >>= 1) plast = max(plast, __shfl_xor(plast, o, NS_WAVE));
+    if (lane == 0) {
+      chunk_sum[wave] = psum;
+      chunk_last[wave] = plast;
     }
   }
   __syncthreads();
-  int tok = s_idx;
-  if (tok == 0x7fffffff) {  // u * total rounded up to the total: the last token that stayed
-    __syncthreads();
-    if (tid == 0) s_idx = -1;
-    __syncthreads();
-    if (last_kept >= 0) atomicMax(&s_idx, last_kept);
-    __syncthreads();
-    tok = s_idx;
-    if (tok < 0) tok = amax;  // nothing stayed (a row of NaN)
+  if (sel < 0) {  // u * total rounded up to the total: the last token that stayed
+    tok = last_all;
+  } else {
+    float run = sel_before, run0 = 0.f;
+    int last_in_chunk = -1;
+    for (int j = 0; j < WAVES; ++j) {
+      if (owner < 0 && run + chunk_sum[j] > target) {
+        owner = j;
+        run0 = run;
+      }
+      run += chunk_sum[j];
+      last_in_chunk = max(last_in_chunk, chunk_last[j]);
+    }
+    if (owner < 0) {  // the sums of the two passes round differently: the passing lies at the chunk's end
+      tok = last_in_chunk;
+    } else if (wave == owner) {
+      run = run0;
+      int last_here = -1;
+      for (int b0 = p0; b0 < p1 && tok < 0; b0 += AHEAD * NS_WAVE) {
+        float p[AHEAD], sum[AHEAD];
+        bool kept[AHEAD];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) p[j] = z[min(b0 + j * NS_WAVE + lane, p1 - 1)];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) {
+          p[j] = weigh(p[j], kept[j]);
+          if (b0 + j * NS_WAVE + lane >= p1) {
+            kept[j] = false;
+            p[j] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) sum[j] = wave_sum(p[j]);  // eight independent chains of lane exchanges
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) {
+          if (tok >= 0) break;
+          const int b = b0 + j * NS_WAVE;
+          const unsigned long long stays = __ballot(kept[j]);
+          if (run + sum[j] > target) {  // the passing lies in these 64 tokens: inclusive sums over the lanes find it
+            float scan = p[j];
+#pragma unroll
+            for (int o = 1; o < NS_WAVE; o <<= 1) {
+              const float t = __shfl_up(scan, o, NS_WAVE);
+              if (lane >= o) scan += t;
+            }
+            const unsigned long long hit = __ballot(kept[j] && run + scan > target);
+            // (the scan and the sum round differently: without a hit the passing is the last token here that stayed)
+            tok = hit ? b + __ffsll((long long)hit) - 1 : b + 63 - __clzll((long long)stays);
+          } else {
+            if (stays) last_here = b + 63 - __clzll((long long)stays);
+            run += sum[j];
+          }
+        }
+      }
+      if (tok < 0) tok = last_here;  // again the rounding: the passing lies at the piece's end
+    }
   }
-  if (tid == 0) {
+  const bool by_first = sel < 0 || owner < 0;  // every thread knows the token; else only the wave that walked does
+  if (by_first ? tid == 0 : (wave == owner && lane == 0)) {
+    if (tok < 0) tok = amax;  // nothing stayed (a row of NaN)
     out_tok[r] = tok;
     out_logprob[r] = z[tok] - lse;
-    out_sample_logprob[r] = z[tok] / T - smax - logf(total);
+    out_sample_logprob[r] = (filtered ? z[tok] / T - smax : (z[tok] - zmax) * inv_t) - logf(total);
   }
 }
 

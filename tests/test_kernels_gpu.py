@@ -585,6 +585,35 @@ def test_sample_greedy_and_temperature():
     assert int(tok[2]) == 100
 
 
+@pytest.mark.parametrize("vocab", [33, 257, 4100, 128256])
+def test_sample_draws_at_other_vocabulary_sizes(vocab):
+    """The inverse CDF is found in two cuts of the vocabulary and a walk: sizes below one cut, off every multiple, and
+    the 8B shape's; uniform numbers at both ends; the draw must be the plain implementation's or its neighbour among the
+    tokens that carry weight (the cumulative sums round differently)."""
+    ops = _ops()
+    torch.manual_seed(vocab)
+    rows = 12
+    z = torch.randn(rows, vocab, device=DEV) * 4
+    z[3, : vocab // 2] = -math.inf  # weightless tokens are never drawn
+    T = torch.tensor([0.5, 0.8, 1.0, 1.0, 0.7, 1.3, 0.9, 1.1, 0.6, 1.0, 2.0, 0.0], device=DEV)
+    u = torch.tensor([0.0, 0.9999999, 0.5, 0.001, 0.25, 0.75, 0.1, 0.9, 0.33, 0.66, 0.999, 0.5], device=DEV)
+    tok, lp, slp = ops.unpack_sample(ops.sample(z, T, u))
+    zc = z.cpu()
+    for r in range(rows):
+        t = float(T[r])
+        if t == 0:
+            assert int(tok[r]) == int(zc[r].argmax())
+            continue
+        ref_lp = pl.processed_logprobs(zc[r], t, 0, 1.0)
+        ref = pl.draw_token(ref_lp, float(u[r]))
+        got = int(tok[r])
+        assert ref_lp[got] > -math.inf
+        cdf = torch.cumsum(torch.exp(ref_lp.double()), 0)
+        assert abs(float(cdf[got]) - float(cdf[ref])) < 1e-4, (r, got, ref)  # no more than rounding apart in the CDF
+        assert abs(float(slp[r]) - float(ref_lp[got])) < 2e-4
+        assert abs(float(lp[r]) - float(torch.log_softmax(zc[r], -1)[got])) < 2e-4
+
+
 def test_sample_top_k_top_p():
     ops = _ops()
     torch.manual_seed(1)
