@@ -485,6 +485,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int hblks = (G + 3) / 4;
     const int ny = a.kv_heads * hblks;
     const int split = blockIdx.x % a.splits, ts = blockIdx.x / a.splits;  // the ranges of a tile start together
+    // Workgroups go round the eight XCDs in the order of blockIdx.x, and each XCD has an L2 of its own.  The key/value
+    // head is the fast index, so with eight of them (or a divisor of eight) an XCD only ever sees one head's keys and
+    // values, and every tile of a prompt re-reads them from that XCD's L2.
     const int y = ts % ny;
     // tiles are listed in the order of the tokens; the last ones see the most keys, so they start first
     const int tile = a.n_tiles - 1 - ts / ny;

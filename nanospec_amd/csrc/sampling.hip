@@ -16,6 +16,9 @@
 #include "common.h"
 
 #define SP_THREADS 1024
+#define SP_CANDIDATES 8192  // tokens near the maximum that the top-k / top-p search keeps in LDS
+#define SP_MARGINS 4        // margins below the maximum that are tried for them, widest first
+__device__ __forceinline__ float sp_margin(int d) { return d == 0 ? 16.f : d == 1 ? 8.f : d == 2 ? 4.f : 2.f; }
 
 // Order-preserving map between floats and unsigned integers.
 __device__ __forceinline__ uint32_t f2ord(float f) {
@@ -38,6 +41,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
   __shared__ float chunk_sum[WAVES];
   __shared__ int chunk_last[WAVES];
   __shared__ int s_idx;
+  __shared__ float cand[SP_CANDIDATES];
   const int r = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (size_t)r * row_stride;
   const bool wide = (((uintptr_t)z) & 15) == 0;
@@ -96,23 +100,85 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
   const float pp = top_p ? top_p[r] : 1.f;
   float cut = -INFINITY;  // tokens with s >= cut stay
   if (k > 0 || pp < 1.f) {
+    // keep(v) = (#{s_j > v} < k) and (mass{s_j > v} <= top_p * total) is monotone in v; the cut is the smallest v (as an
+    // ordered bit pattern) for which it holds.  Each probe of the bisection is a sum over the tokens above v.  Where the cut
+    // lies among the few tokens within a margin of the maximum, those are first gathered into LDS (in an order that is
+    // the same in every run) and the probes only walk them; otherwise the probes walk the whole row.
     float tot = 0.f;
-    for (int i = tid; i < vocab; i += SP_THREADS) tot += expf(z[i] / T - smax);
+    float cnt_m[SP_MARGINS], mass_m[SP_MARGINS];
+#pragma unroll
+    for (int d = 0; d < SP_MARGINS; ++d) cnt_m[d] = mass_m[d] = 0.f;
+    for (int i = tid; i < vocab; i += SP_THREADS) {
+      const float sv = z[i] / T;
+      const float e = expf(sv - smax);
+      tot += e;
+#pragma unroll
+      for (int d = 0; d < SP_MARGINS; ++d)
+        if (sv > smax - sp_margin(d)) { cnt_m[d] += 1.f; mass_m[d] += e; }
+    }
     tot = block_sum(tot, scratch);
-    // smallest ordered key x with keep(ord2f(x)); keep(max) holds (nothing is above the maximum)
-    uint32_t lo = 0u, hi = f2ord(smax);
+    int use = -1;  // the widest margin whose tokens fit the LDS array
+    float cnt_u = 0.f, mass_u = 0.f;
+#pragma unroll
+    for (int d = 0; d < SP_MARGINS; ++d) {
+      const float c = block_sum(cnt_m[d], scratch), m = block_sum(mass_m[d], scratch);
+      if (use < 0 && c <= (float)SP_CANDIDATES) { use = d; cnt_u = c; mass_u = m; }
+    }
+    auto keep = [&](float cnt, float mass) { return (k <= 0 || cnt < (float)k) && (mass / tot <= pp); };
+    uint32_t lo = 0u, hi = f2ord(smax);  // keep(max) holds: nothing is above the maximum
+    bool gathered = false;
+    if (use >= 0) {
+      const float tau = smax - sp_margin(use);
+      if (keep(cnt_u, mass_u)) {
+        hi = f2ord(tau);  // the cut lies at or below the margin: probe the whole row, from there down
+      } else {
+        lo = f2ord(tau) + 1;  // the cut lies above it, among the gathered tokens
+        gathered = true;
+      }
+    }
+    int n_cand = 0;
+    if (gathered) {
+      // thread t gathers its tokens t, t + 1024, ... in that order behind those of the threads before it
+      int mine_n = 0;
+      const float tau = smax - sp_margin(use);
+      for (int i = tid; i < vocab; i += SP_THREADS) mine_n += (z[i] / T > tau) ? 1 : 0;
+      int incl = mine_n;
+#pragma unroll
+      for (int o = 1; o < NS_WAVE; o <<= 1) {
+        const int t = __shfl_up(incl, o, NS_WAVE);
+        if ((tid & (NS_WAVE - 1)) >= o) incl += t;
+      }
+      __syncthreads();
+      if ((tid & (NS_WAVE - 1)) == NS_WAVE - 1) chunk_last[tid / NS_WAVE] = incl;
+      __syncthreads();
+      int at = incl - mine_n;
+      for (int j = 0; j < tid / NS_WAVE; ++j) at += chunk_last[j];
+      for (int j = 0; j < WAVES; ++j) n_cand += chunk_last[j];
+      for (int i = tid; i < vocab; i += SP_THREADS) {
+        const float sv = z[i] / T;
+        if (sv > tau && at < SP_CANDIDATES) cand[at++] = sv;
+      }
+      n_cand = min(n_cand, SP_CANDIDATES);
+      __syncthreads();
+    }
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo) / 2;
       const float v = ord2f(mid);
       float cnt = 0.f, mass = 0.f;
-      for (int i = tid; i < vocab; i += SP_THREADS) {
-        const float s = z[i] / T;
-        if (s > v) { cnt += 1.f; mass += expf(s - smax); }
+      if (gathered) {
+        for (int i = tid; i < n_cand; i += SP_THREADS) {
+          const float sv = cand[i];
+          if (sv > v) { cnt += 1.f; mass += expf(sv - smax); }
+        }
+      } else {
+        for (int i = tid; i < vocab; i += SP_THREADS) {
+          const float sv = z[i] / T;
+          if (sv > v) { cnt += 1.f; mass += expf(sv - smax); }
+        }
       }
       cnt = block_sum(cnt, scratch);
       mass = block_sum(mass, scratch);
-      const bool keep = (k <= 0 || cnt < (float)k) && (mass / tot <= pp);
-      if (keep) hi = mid; else lo = mid + 1;
+      if (keep(cnt, mass)) hi = mid; else lo = mid + 1;
     }
     cut = ord2f(lo);
   }
