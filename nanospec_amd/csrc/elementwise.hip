@@ -357,7 +357,29 @@ __global__ void rope_kv_vec_kernel(T* __restrict__ qkv, int row_stride, const in
     const int h = u / plain, d0 = rot + (u - h * plain) * V;
     *reinterpret_cast<vec_t*>(kdst + (size_t)h * page_size * hd + d0) = *reinterpret_cast<const vec_t*>(krow + h * hd + d0);
   }
-  for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x) vdst[(size_t)e * page_size] = vrow[e];
+  // V pages hold a channel's tokens side by side.  The tokens of a request stand in the batch one after the other at
+  // rising positions, so up to V of them fall into one aligned run of V slots of a page: the first of them writes
+  // the run for all, a full run as one 16-byte store per channel instead of V stores of one element each.
+  const int n_tokens = gridDim.x;
+  const int req = token_req[t];
+  int cnt = 1;
+  if (page_size % V == 0) {
+    const bool first = t == 0 || token_req[t - 1] != req;
+    if (!first && pos % V != 0) return;  // an earlier token of the run writes this one's values
+    const int room = min(V - pos % V, n_tokens - t);
+    while (cnt < room && token_req[t + cnt] == req) ++cnt;
+  }
+  if (cnt == V) {
+    for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x) {
+      vec_t val;
+#pragma unroll
+      for (int i = 0; i < V; ++i) val[i] = vrow[(size_t)i * row_stride + e];
+      *reinterpret_cast<vec_t*>(vdst + (size_t)e * page_size) = val;
+    }
+  } else {
+    for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x)
+      for (int i = 0; i < cnt; ++i) vdst[(size_t)e * page_size + i] = vrow[(size_t)i * row_stride + e];
+  }
 }
 
 extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions, const int* token_req,
@@ -369,7 +391,7 @@ extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions,
   const int work = heads * (rot / 2) > kv_heads * hd ? heads * (rot / 2) : kv_heads * hd;
   const int threads = work >= 1024 ? 1024 : work >= 512 ? 512 : 256;
   const int vlen = dtype == NS_DTYPE_F32 ? 4 : 8;
-  const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache) & 15) == 0 && row_stride % vlen == 0 && (rot / 2) % vlen == 0 &&
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0 && row_stride % vlen == 0 && (rot / 2) % vlen == 0 &&
                        (hd - rot) % vlen == 0 && hd % vlen == 0 && rot > 0;
   if (aligned) {
     const int vthreads = threads >= 512 ? 256 : threads;
