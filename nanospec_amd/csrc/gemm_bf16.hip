@@ -23,6 +23,13 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 #define EPI_SILU_MUL 1
 #define EPI_ROPE_KV 2
 #define EPI_RESID_NORM 3
+#define EPI_GATED_HALF 4
+// EPI_GATED_HALF is EPI_SILU_MUL with half the work per workgroup: the 16 rows of a workgroup's matrix instruction are 8
+// rows of the gate matrix and the same 8 rows of the up matrix (a lane is free to take its 16 bytes from any row of
+// either tiled matrix), placed so that a gate row's sum and its up row's sum come out in the same lane.  Twice as many
+// workgroups, each streaming half as much: a compute unit streams at a fixed rate, so a product takes as long as the
+// compute unit with the most workgroups, and 14,336 rows are 3.5 workgroups per compute unit of the one kind (as slow as 4)
+// and 7 of the other.
 
 // What the q/k/v epilogue needs: the rows of the stacked [q; k; v] matrix were permuted at load time so that a
 // workgroup's 16 rows are, for the rotary part of a q or k head, 8 channels j and their partners j + rot/2, and
@@ -71,7 +78,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
   __shared__ float rinv_s[MT * 16];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in a wave's lanes
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int tile = EPI == EPI_GATED_HALF ? blockIdx.x >> 1 : blockIdx.x;  // the stored row tile(s) this workgroup reads
+  const int n0 = tile * 16;
   const int KT = (K + 127) / 128;
   // What the epilogue needs besides the sums is asked for now and used after the weights have streamed.
   // Consumer: wave v takes rows v, v + WAVES, ...; its lanes take the producer's workgroups in turn.
@@ -100,7 +108,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
       wnext_pre[i] = (float)nl.w_next[n];
     }
   }
-  const bf16_t* wbase = wt + (size_t)blockIdx.x * KT * 2048 + lane * 8;
+  // EPI_GATED_HALF: rows 4 q + {0, 1} of the instruction are gate rows 8 h + 2 q + {0, 1} of the tile, rows 4 q + {2, 3} the
+  // same rows of the up matrix (h = which half of the tile); the sums of row 4 q + j come out in lane group q, element j.
+  const int src_row = EPI == EPI_GATED_HALF ? 8 * (blockIdx.x & 1) + 2 * (r >> 2) + (r & 1) : r;
+  const bf16_t* wsrc = (EPI == EPI_GATED_HALF && (r & 2)) ? wt2 : wt;
+  const bf16_t* wbase = wsrc + (size_t)tile * KT * 2048 + (16 * g + src_row) * 8;
   const bf16_t* w2base = EPI == EPI_SILU_MUL ? wt2 + (size_t)blockIdx.x * KT * 2048 + lane * 8 : nullptr;
   const bf16_t* xrow[MT];
 #pragma unroll
@@ -279,6 +291,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
     }
     return;
   }
+  if (EPI == EPI_GATED_HALF) {
+    for (int e = threadIdx.x; e < MT * 128; e += WAVES * 64) {
+      const int mt = e >> 7, l = (e & 127) >> 1, j = e & 1;  // lane l of the sums holds gate at j, up at 2 + j
+      const int n = n0 + 8 * (blockIdx.x & 1) + 2 * (l >> 4) + j, m = mt * 16 + (l & 15);
+      if (n >= N || m >= M) continue;
+      float s = 0.f, u = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) {
+        s += red[wv][mt][l * 4 + j];
+        u += red[wv][mt][l * 4 + 2 + j];
+      }
+      if (nl.ssq_in) {
+        s *= rinv_s[m];
+        u *= rinv_s[m];
+      }
+      out[(size_t)m * out_stride + n] = (OutT)(s / (1.f + expf(-s)) * u);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < MT * 256; e += WAVES * 64) {
     const int mt = e >> 8, le = e & 255;
     const int l = le >> 2, j = le & 3;
@@ -309,6 +340,9 @@ static int launch_tiled(void* out, const void* x, const void* w, const void* w2,
   if (epi == EPI_SILU_MUL) {
     if (out_f32) return NS_ERR_UNSUPPORTED;
     gemm_tiled_kernel<MT, WAVES, EPI_SILU_MUL, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, w2b, M, N, K, x_stride, out_stride, rk, nl);
+  } else if (epi == EPI_GATED_HALF) {
+    if (out_f32 || MT != 1) return NS_ERR_UNSUPPORTED;
+    gemm_tiled_kernel<1, WAVES, EPI_GATED_HALF, bf16_t><<<2 * grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, w2b, M, N, K, x_stride, out_stride, rk, nl);
   } else if (epi == EPI_RESID_NORM) {
     if (out_f32 || MT != 1) return NS_ERR_UNSUPPORTED;
     gemm_tiled_kernel<1, WAVES, EPI_RESID_NORM, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk, nl);
@@ -328,7 +362,7 @@ static int tiled_dispatch(void* out, const void* x, const void* wt, const void* 
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K) return NS_ERR_BAD_ARG;
   if (epi != EPI_ROPE_KV && epi != EPI_RESID_NORM && out_stride < N) return NS_ERR_BAD_ARG;
   if (nl.ssq_in && (nl.parts_in <= 0 || M > 16)) return NS_ERR_BAD_ARG;
-  if (epi == EPI_SILU_MUL && !wt2) return NS_ERR_BAD_ARG;
+  if ((epi == EPI_SILU_MUL || epi == EPI_GATED_HALF) && !wt2) return NS_ERR_BAD_ARG;
   const int mt = (M + 15) / 16;
 #define NS_TILED(MTV)                                                                                               \
   case MTV:                                                                                                         \
@@ -350,7 +384,7 @@ static int tiled_dispatch(void* out, const void* x, const void* wt, const void* 
 extern "C" int ns_gemm_tiled_bf16(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
                                   int x_stride, int out_stride, int epi, int out_f32, int waves, const float* ssq_in,
                                   int parts_in, int norm_dim, float eps, hipStream_t stream) {
-  if (epi != EPI_STORE && epi != EPI_SILU_MUL) return NS_ERR_BAD_ARG;
+  if (epi != EPI_STORE && epi != EPI_SILU_MUL && epi != EPI_GATED_HALF) return NS_ERR_BAD_ARG;
   RopeKvParams rk = {};
   NormLink nl = {};
   nl.ssq_in = ssq_in; nl.parts_in = parts_in; nl.inv_dim = norm_dim > 0 ? 1.f / (float)norm_dim : 0.f; nl.eps = eps;

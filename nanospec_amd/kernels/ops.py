@@ -295,10 +295,15 @@ def _prenorm_args(pre: "PreNormed | None", m: int, what: str):
     return _ptr(pre.ssq), c_int(pre.ssq.shape[1]), c_int(pre.dim), c_float(pre.eps)
 
 
+GATED_HALF_ROWS = 4  # up to this many rows the gated product runs half a row tile of each matrix per workgroup (with more,
+#                      reading x in twice as many workgroups costs what the even spread gains)
+
+
 def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
-                 out_f32: bool = False, waves: int = 0) -> torch.Tensor:
+                 out_f32: bool = False, waves: int = 0, halves: bool | None = None) -> torch.Tensor:
     """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T).  ``x`` may be a
-    ``PreNormed`` (at most 16 rows)."""
+    ``PreNormed`` (at most 16 rows).  ``halves`` (with ``w2``, at most 16 rows): a workgroup takes 8 rows of each matrix
+    instead of 16, which spreads a number of row tiles that is no multiple of the compute units evenly; None: by rows."""
     pre = x if isinstance(x, PreNormed) else None
     if pre is not None:
         x = pre.x
@@ -316,9 +321,12 @@ def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight 
         raise KernelRefused("linear_tiled: w2 must match w")
     if waves == 0:  # with more than 8 rows eight waves were never behind four at the shapes measured
         waves = 8 if w.k >= 8192 or ((w.n // 16 < 512 or m > 8) and w.k >= 2048) else 4
+    if halves is None:
+        halves = m <= GATED_HALF_ROWS
+    epi = 0 if w2 is None else (4 if halves and m <= 16 and not out_f32 else 1)
     _check(build.core().ns_gemm_tiled_bf16(_ptr(out), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None), c_int(m),
                                            c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
-                                           c_int(1 if w2 is not None else 0), c_int(1 if out_f32 else 0), c_int(waves),
+                                           c_int(epi), c_int(1 if out_f32 else 0), c_int(waves),
                                            *_prenorm_args(pre, m, "linear_tiled"), _stream()),
            "linear_tiled")
     return out

@@ -108,6 +108,23 @@ def test_linear_tiled(m, n, k):
         torch.testing.assert_close(part.cpu(), ref[:, 16:48], rtol=1e-4, atol=1e-3 * math.sqrt(k))
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064), (14336, 512)])
+def test_gated_product_in_half_tiles(m, n, k):
+    """silu(x Wg^T) * (x Wu^T) with 8 rows of each matrix per workgroup: the same bits as with 16, at sizes off the tile."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m + 3, k + 8, dtype=torch.bfloat16, device=DEV)[:m, :k]
+    wg, wu = (torch.randn(n, k, dtype=torch.bfloat16, device=DEV) * 0.3 for _ in range(2))
+    tg, tu = ops.TiledWeight(wg), ops.TiledWeight(wu)
+    g, u = x.cpu().float() @ wg.cpu().float().T, x.cpu().float() @ wu.cpu().float().T
+    for waves in (2, 4, 8):
+        whole = ops.linear_tiled(x, tg, w2=tu, waves=waves, halves=False)
+        halves = ops.linear_tiled(x, tg, w2=tu, waves=waves, halves=True)
+        assert torch.equal(whole, halves)
+        assert ulps_of_row_max(halves.cpu(), g * torch.sigmoid(g) * u).max() <= 1.0
+
+
 @pytest.mark.parametrize("m", [17, 33, 48, 64, 5])
 @pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064), (4096, 14336)])
 def test_linear_wide(m, n, k):
