@@ -40,6 +40,11 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
   const int split = blockIdx.y;
   const int per = (KT + ksplit - 1) / ksplit;
   const int kt0 = split * per, kt1 = min(KT, kt0 + per);
+  // more than MT * 16 rows of x: blockIdx.z takes them MT * 16 at a time (every block of rows reads the weights again)
+  const int m_base = blockIdx.z * (MT * 16);
+  const int m_total = M;
+  x += (size_t)m_base * x_stride;
+  M = min(MT * 16, M - m_base);
 
   const bf16_t* wbase = wt + (size_t)(has_rows ? rt : 0) * KT * 2048 + lane * 8;
   const bf16_t* w2base = NACC == 2 ? wt2 + (size_t)(has_rows ? rt : 0) * KT * 2048 + lane * 8 : nullptr;
@@ -143,6 +148,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
       for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r, n = (rt + t) * 16 + g * 4;
         if (m >= M || !tile_ok[t]) continue;
+        const int mg = m_base + m;
         f32x4 v = acc[0][t][mt];
         if (NACC == 2) {
 #pragma unroll
@@ -151,8 +157,8 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if (n + j < N) {
-            if (out_f32) ((float*)direct_out)[(size_t)m * out_stride + n + j] = v[j];
-            else ((bf16_t*)direct_out)[(size_t)m * out_stride + n + j] = (bf16_t)v[j];
+            if (out_f32) ((float*)direct_out)[(size_t)mg * out_stride + n + j] = v[j];
+            else ((bf16_t*)direct_out)[(size_t)mg * out_stride + n + j] = (bf16_t)v[j];
           }
       }
     return;
@@ -165,7 +171,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ part
       for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r, n = (rt + t) * 16 + g * 4;
         if (m >= M || !tile_ok[t]) continue;
-        float* dst = partial + ((size_t)(a * ksplit + split) * M + m) * N + n;
+        float* dst = partial + ((size_t)(a * ksplit + split) * m_total + m_base + m) * N + n;
         if (n + 3 < N && (N & 3) == 0) {
           *reinterpret_cast<f32x4*>(dst) = acc[a][t][mt];
         } else {
@@ -244,6 +250,47 @@ extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, cons
     case 7: st = launch_wide_tall<7>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
     default: st = launch_wide_tall<8>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
   }
+  if (st != NS_OK || direct) return st;
+  if (defer) return epi == 0 ? NS_OK : NS_ERR_BAD_ARG;
+  const size_t total = (size_t)M * N;
+  const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+  if (epi == 1)
+    gemm_wide_reduce_kernel<bf16_t, 1><<<blocks, 256, 0, stream>>>((bf16_t*)out, part, M, N, out_stride, ksplit);
+  else if (out_f32)
+    gemm_wide_reduce_kernel<float, 0><<<blocks, 256, 0, stream>>>((float*)out, part, M, N, out_stride, ksplit);
+  else
+    gemm_wide_reduce_kernel<bf16_t, 0><<<blocks, 256, 0, stream>>>((bf16_t*)out, part, M, N, out_stride, ksplit);
+  return ns_launch_status();
+}
+
+// Any number of rows, 128 at a time over blockIdx.z, with `nt` row tiles of w per wave (2 or 4; 1 or 2 with wt2): each
+// fragment of x read from LDS then serves nt (2 nt with wt2) matrix instructions, which is what many rows need.  Every
+// block of 128 rows reads the weights again (from the caches, if the matrix fits them).  For models whose weights are
+// kept in the tiled layout only.  Arguments as ns_gemm_wide_bf16.
+extern "C" int ns_gemm_rows_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
+                                 int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer,
+                                 hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
+  if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
+  const int KT = (K + 127) / 128;
+  if (ksplit < 1 || ksplit > KT || ksplit > 65535 || (ksplit > 1 && !workspace)) return NS_ERR_BAD_ARG;
+  if (wt2 ? (nt != 1 && nt != 2) : (nt != 2 && nt != 4)) return NS_ERR_BAD_ARG;
+  const int m_blocks = (M + 127) / 128;
+  if (m_blocks > 65535) return NS_ERR_BAD_ARG;
+  const int row_tiles = (N + 15) / 16;
+  dim3 grid((row_tiles + 4 * nt - 1) / (4 * nt), ksplit, m_blocks);
+  float* part = (float*)workspace;
+  void* direct = ksplit == 1 ? out : nullptr;
+  const bf16_t *xp = (const bf16_t*)x, *w1 = (const bf16_t*)wt, *w2 = (const bf16_t*)wt2;
+  if (wt2 && nt == 2)
+    gemm_wide_kernel<8, 2, 2><<<grid, 256, 0, stream>>>(part, xp, w1, w2, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+  else if (wt2)
+    gemm_wide_kernel<8, 2, 1><<<grid, 256, 0, stream>>>(part, xp, w1, w2, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+  else if (nt == 4)
+    gemm_wide_kernel<8, 1, 4><<<grid, 256, 0, stream>>>(part, xp, w1, nullptr, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+  else
+    gemm_wide_kernel<8, 1, 2><<<grid, 256, 0, stream>>>(part, xp, w1, nullptr, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+  int st = ns_launch_status();
   if (st != NS_OK || direct) return st;
   if (defer) return epi == 0 ? NS_OK : NS_ERR_BAD_ARG;
   const size_t total = (size_t)M * N;

@@ -408,6 +408,47 @@ def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, 
     return PartialSums(workspace, ksplit, m, w.n, x.dtype) if defer else out
 
 
+def rows_plan(n: int, k: int, rows: int, gated: bool = False) -> tuple[int, int]:
+    """(ranges K is cut into, 16-row tiles per wave) of ``linear_rows``: the most tiles per wave, then ranges of K until
+    the workgroups fill the GPU, with at least eight k tiles of 128 per range."""
+    nt = 2 if gated else 4
+    groups = -(-n // (64 * nt)) * -(-rows // 128)
+    k_tiles = -(-k // 128)
+    return max(1, min(16, k_tiles // 8, 256 // groups)), nt
+
+
+def linear_rows(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
+                out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0):
+    """bfloat16 x @ w.T for any number of rows from a tiled weight: the kernel of ``linear_wide`` over blocks of 128 rows,
+    with ``nt`` (2 or 4; 1 or 2 with ``w2``) row tiles of the weight per wave.  For models that keep the tiled layout only:
+    the platform's library is twice as fast where the plain layout is there for it.  Arguments as ``linear_wide``."""
+    _gpu(x, out, workspace)
+    if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k, x.shape[0]):
+        raise KernelRefused(f"linear_rows takes bfloat16 x [rows, {w.k}] with an inner size that is a multiple of 8; got "
+                            f"{tuple(x.shape)} {x.dtype}")
+    m = x.shape[0]
+    want = torch.float32 if out_f32 else x.dtype
+    plan = rows_plan(w.n, w.k, m, w2 is not None)
+    ksplit, nt = ksplit or plan[0], nt or plan[1]
+    if out is None:
+        out = torch.empty((m, w.n), dtype=want, device=x.device)
+    if out.shape != (m, w.n) or out.dtype != want or out.stride(1) != 1:
+        raise KernelRefused("linear_rows: out has the wrong shape or dtype")
+    if w2 is not None and (w2.n != w.n or w2.k != w.k or out_f32):
+        raise KernelRefused("linear_rows: w2 must match w and the gated result is bfloat16")
+    need = (2 if w2 is not None else 1) * ksplit * m * w.n if ksplit > 1 else 0
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+    if need and (workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous()):
+        raise KernelRefused("linear_rows: workspace too small")
+    _check(build.core().ns_gemm_rows_bf16(_ptr(out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data),
+                                          _ptr(w2.data if w2 is not None else None), c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)),
+                                          c_int(out.stride(0)), c_int(1 if w2 is not None else 0),
+                                          c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), c_int(0), _stream()),
+           "linear_rows")
+    return out
+
+
 def qkv_rope_row_order(heads: int, kv_heads: int, head_dim: int, rotary_dim: int) -> torch.Tensor:
     """The row order of a stacked [q; k; v] matrix for ``linear_qkv_rope``: per head 16-row tiles; in the rotary part of a
     q or k head a tile holds 8 channels j and their partners j + rotary_dim/2, elsewhere 16 consecutive channels."""

@@ -126,6 +126,10 @@ class LinearWeight:
             return torch.matmul(x, self._plain_t) if out is None else torch.matmul(x, self._plain_t, out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
+        if m > ops.WIDE_TALL_ROWS:  # only the tiled layout is kept: blocks of 128 rows through the hand-written kernel
+            ksplit, nt = ops.rows_plan(self.n, self.k, m)
+            ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
+            return ops.linear_rows(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
         ksplit, nt = ops.wide_plan(self.n, self.k)
         ws = arena.take((ksplit * ops.SKINNY_MAX_ROWS * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
         for s in range(0, m, ops.SKINNY_MAX_ROWS):
@@ -161,6 +165,9 @@ class GatedWeights:
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
+        if fast and self.stacked is None and m > ops.WIDE_TALL_ROWS:
+            # only the tiled layout is kept: blocks of 128 rows through the hand-written kernel, activation in the same pass
+            return ops.linear_rows(x, self.tiled[0], w2=self.tiled[1], out=out, ksplit=1, nt=2)
         if fast and (m <= ops.SKINNY_MAX_ROWS or self.stacked is None):
             # 17 to 64 rows: the second hand-written kernel, one range of K, so that the activation is applied in the same
             # pass (measured ahead of the library's product plus the activation kernel)

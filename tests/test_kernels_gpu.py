@@ -330,6 +330,33 @@ def test_linear_wide_up_to_128_rows(m, n, k):
         ops.linear_wide(torch.randn(129, k, dtype=torch.bfloat16, device=DEV), wt)
 
 
+@pytest.mark.parametrize("m", [129, 300, 1031])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 2056), (4096, 1024)])
+def test_linear_rows(m, n, k):
+    """Any number of rows in blocks of 128 (what a model that keeps the tiled layout only runs its prompts through): every
+    count of row tiles per wave and several counts of ranges, sizes off every tile, the gated form, 32-bit results."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m + 3, k + 8, dtype=torch.bfloat16, device=DEV)[:m, :k]
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    wt, wt2 = ops.TiledWeight(w), ops.TiledWeight(w2)
+    ref = x.cpu().float() @ w.cpu().float().T
+    k_tiles = -(-k // 128)
+    for nt in (2, 4):
+        for ks in sorted({1, min(3, k_tiles), 0}):
+            out = ops.linear_rows(x, wt, out_f32=True, ksplit=ks, nt=nt if ks else 0)
+            torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
+    assert ulps_of_row_max(ops.linear_rows(x, wt).cpu(), ref).max() <= 1.0
+    u = x.cpu().float() @ w2.cpu().float().T
+    for nt in (1, 2):
+        for ks in (1, min(2, k_tiles)):
+            act = ops.linear_rows(x, wt, w2=wt2, ksplit=ks, nt=nt)
+            assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0
+    with pytest.raises(ops.KernelRefused):
+        ops.linear_rows(x, wt, nt=1)
+
+
 @pytest.mark.parametrize("m", [17, 40, 64, 97, 128])
 @pytest.mark.parametrize("hidden,inner,ksplit", [(136, 1024, 4), (4096, 1024, 2), (72, 512, 3)])
 def test_ranges_of_a_product_added_by_the_norm_that_reads_them(m, hidden, inner, ksplit):
