@@ -136,7 +136,11 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
 
   int kb0 = whi > 0 ? wlo / 32 : 0, kb1 = whi > 0 ? (whi + 31) / 32 : 0;
   if (a.splits > 1) {
-    const int per = (kb1 - kb0 + a.splits - 1) / a.splits;
+    // More than 16 ranges (a launch of few tiles, made for long rows of keys) are only used from 8,192 keys on: below
+    // that the ranges beyond the sixteenth stay empty and the others are as long as a launch of 16 would make them.
+    const int blocks = kb1 - kb0;
+    const int ranges = (a.splits > 16 && blocks < 256) ? 16 : a.splits;
+    const int per = (blocks + ranges - 1) / ranges;
     kb0 = kb0 + split * per;
     kb1 = min(kb1, kb0 + per);
   }

@@ -113,8 +113,11 @@ class StepContext:
                 hp *= 2
             # decode is bound by the latency of each wave's chain of loads: the four waves of a workgroup share a tile, and
             # the keys are cut into ranges until about a thousand waves are at work
+            # (up to 32 ranges where requests may reach 8,192 keys and the tiles are few, a single request say: at 131,072
+            # keys 86 against 132 us a layer; the kernel leaves the ranges beyond the sixteenth empty for shorter rows,
+            # and where no request can be that long they are not launched: they would cost a captured step 1%)
             items = lay.Td * kv_heads * -(-group // hp)
-            splits = max(1, min(16, 1024 // (4 * items)))
+            splits = max(1, min(32 if self.max_kv_len >= 8192 else 16, 1024 // (4 * items)))
             if not self.fixed_splits:
                 splits = max(1, min(splits, -(-self.max_kv_len // 256)))
             ws = None
