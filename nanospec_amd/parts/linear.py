@@ -120,6 +120,11 @@ class LinearWeight:
             ksplit, nt = ops.wide_plan(self.n, self.k)
             ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
             return ops.linear_wide(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
+        if self.tiled is not None and m <= ops.WIDE_TALL_ROWS and self.n <= WIDE_MAX_N:
+            # 65 to 128 rows of a narrow product (the last layer's down-projection, which no norm inside the layer loop follows)
+            ksplit, nt = ops.wide_plan(self.n, self.k, m)
+            ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
+            return ops.linear_wide(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
         if self.plain is not None and (not out_f32 or self.tiled is None):
             if out_f32:
                 return ops.linear_generic(x, self.plain, out=out, out_f32=True)
