@@ -517,7 +517,9 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
             hp *= 2
         splits = force_splits or 3
         cols = len(dt) * (16 // hp) * heads
-        ws = (torch.empty(cols * splits * hd, dtype=torch.float32, device=DEV), torch.empty(cols * splits * 2, dtype=torch.float32, device=DEV))
+        # filled with NaN: a range (an empty one, say: with more than 16 the later ones are, below 8,192 keys) that is read
+        # without having been written shows
+        ws = (torch.full((cols * splits * hd,), float("nan"), device=DEV), torch.full((cols * splits * 2,), float("nan"), device=DEV))
         ops.attention_mfma(q, out, k, v, i32(dt), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=hp,
                            splits=splits, workspace=ws if splits > 1 else None, coop=coop)
     return out
