@@ -29,19 +29,31 @@ template <int MT, int NACC, int NT>
 __global__ __launch_bounds__(256) void gemm_wide_kernel(float* __restrict__ partial, const bf16_t* __restrict__ x,
                                                         const bf16_t* __restrict__ wt, const bf16_t* __restrict__ wt2,
                                                         int M, int N, int K, int x_stride, int ksplit,
-                                                        void* __restrict__ direct_out, int out_stride, int out_f32) {
+                                                        void* __restrict__ direct_out, int out_stride, int out_f32,
+                                                        int n_groups, int m_blocks) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][WIDE_XROW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int KT = (K + 127) / 128;
   const int row_tiles = (N + 15) / 16;
-  const int rt = (blockIdx.x * 4 + wave) * NT;  // first of this wave's row tiles
+  // n_groups > 0 (many rows): the launch is one row of workgroups, which go round the eight XCDs in launch order; each XCD
+  // takes a contiguous share of the (group of weight rows, block of x rows) pairs, blocks of x fastest, so that the few
+  // groups of weight rows it works on at a time stay in its own L2 while the blocks of x pass through.
+  int bx = blockIdx.x, bz = blockIdx.z;
+  if (n_groups > 0) {
+    const int total = n_groups * m_blocks, per = (total + 7) / 8;
+    const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    if (t >= total) return;
+    bx = t / m_blocks;
+    bz = t - bx * m_blocks;
+  }
+  const int rt = (bx * 4 + wave) * NT;  // first of this wave's row tiles
   const bool has_rows = rt < row_tiles;
   const int split = blockIdx.y;
   const int per = (KT + ksplit - 1) / ksplit;
   const int kt0 = split * per, kt1 = min(KT, kt0 + per);
   // more than MT * 16 rows of x: blockIdx.z takes them MT * 16 at a time (every block of rows reads the weights again)
-  const int m_base = blockIdx.z * (MT * 16);
+  const int m_base = bz * (MT * 16);
   const int m_total = M;
   x += (size_t)m_base * x_stride;
   M = min(MT * 16, M - m_base);
@@ -205,13 +217,13 @@ static int launch_wide(float* partial, const bf16_t* x, const bf16_t* wt, const 
   const int row_tiles = (N + 15) / 16;
   dim3 grid((row_tiles + 4 * nt - 1) / (4 * nt), ksplit);
   if (wt2 && nt == 2)
-    gemm_wide_kernel<MT, 2, 2><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
+    gemm_wide_kernel<MT, 2, 2><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32, 0, 0);
   else if (wt2)
-    gemm_wide_kernel<MT, 2, 1><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
+    gemm_wide_kernel<MT, 2, 1><<<grid, 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32, 0, 0);
   else if (nt == 2)
-    gemm_wide_kernel<MT, 1, 2><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
+    gemm_wide_kernel<MT, 1, 2><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32, 0, 0);
   else
-    gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
+    gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32, 0, 0);
   return ns_launch_status();
 }
 
@@ -221,7 +233,7 @@ static int launch_wide_tall(float* partial, const bf16_t* x, const bf16_t* wt, i
                             void* direct_out, int out_stride, int out_f32, hipStream_t stream) {
   const int row_tiles = (N + 15) / 16;
   dim3 grid((row_tiles + 3) / 4, ksplit);
-  gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32);
+  gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32, 0, 0);
   return ns_launch_status();
 }
 
@@ -278,18 +290,19 @@ extern "C" int ns_gemm_rows_bf16(void* out, void* workspace, const void* x, cons
   const int m_blocks = (M + 127) / 128;
   if (m_blocks > 65535) return NS_ERR_BAD_ARG;
   const int row_tiles = (N + 15) / 16;
-  dim3 grid((row_tiles + 4 * nt - 1) / (4 * nt), ksplit, m_blocks);
+  const int n_groups = (row_tiles + 4 * nt - 1) / (4 * nt);
+  dim3 grid(8 * ((n_groups * m_blocks + 7) / 8), ksplit, 1);
   float* part = (float*)workspace;
   void* direct = ksplit == 1 ? out : nullptr;
   const bf16_t *xp = (const bf16_t*)x, *w1 = (const bf16_t*)wt, *w2 = (const bf16_t*)wt2;
   if (wt2 && nt == 2)
-    gemm_wide_kernel<8, 2, 2><<<grid, 256, 0, stream>>>(part, xp, w1, w2, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+    gemm_wide_kernel<8, 2, 2><<<grid, 256, 0, stream>>>(part, xp, w1, w2, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, n_groups, m_blocks);
   else if (wt2)
-    gemm_wide_kernel<8, 2, 1><<<grid, 256, 0, stream>>>(part, xp, w1, w2, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+    gemm_wide_kernel<8, 2, 1><<<grid, 256, 0, stream>>>(part, xp, w1, w2, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, n_groups, m_blocks);
   else if (nt == 4)
-    gemm_wide_kernel<8, 1, 4><<<grid, 256, 0, stream>>>(part, xp, w1, nullptr, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+    gemm_wide_kernel<8, 1, 4><<<grid, 256, 0, stream>>>(part, xp, w1, nullptr, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, n_groups, m_blocks);
   else
-    gemm_wide_kernel<8, 1, 2><<<grid, 256, 0, stream>>>(part, xp, w1, nullptr, M, N, K, x_stride, ksplit, direct, out_stride, out_f32);
+    gemm_wide_kernel<8, 1, 2><<<grid, 256, 0, stream>>>(part, xp, w1, nullptr, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, n_groups, m_blocks);
   int st = ns_launch_status();
   if (st != NS_OK || direct) return st;
   if (defer) return epi == 0 ? NS_OK : NS_ERR_BAD_ARG;
