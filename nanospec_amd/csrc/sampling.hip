@@ -187,14 +187,14 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(int* __restrict__ ou
   // stays of it, its lanes reading neighbouring tokens; then the chunk in which the running sum passes u * total is found.
   const bool filtered = cut > -INFINITY;
   const float inv_t = 1.f / T;
-  // what a token weighs and whether it stays; without a cut everything but NaN stays and the weight needs no division
+  // what a token weighs and whether it stays; without a cut everything finite stays and the weight needs no division
   auto weigh = [&](float v, bool& kept) -> float {
     if (filtered) {
       const float sv = v / T;  // the very expression whose values the cut was found among
       kept = sv >= cut;
       return kept ? expf(sv - smax) : 0.f;
     }
-    kept = v == v;
+    kept = v > -INFINITY;  // neither NaN nor a token that was masked out
     return kept ? __expf((v - zmax) * inv_t) : 0.f;
   };
   const int lane = tid & (NS_WAVE - 1), wave = tid / NS_WAVE;

@@ -641,6 +641,7 @@ def test_sample_draws_at_other_vocabulary_sizes(vocab):
     rows = 12
     z = torch.randn(rows, vocab, device=DEV) * 4
     z[3, : vocab // 2] = -math.inf  # weightless tokens are never drawn
+    z[1, vocab - vocab // 3 :] = -math.inf  # ... nor when u * total rounds up to the total and the last token is taken
     T = torch.tensor([0.5, 0.8, 1.0, 1.0, 0.7, 1.3, 0.9, 1.1, 0.6, 1.0, 2.0, 0.0], device=DEV)
     u = torch.tensor([0.0, 0.9999999, 0.5, 0.001, 0.25, 0.75, 0.1, 0.9, 0.33, 0.66, 0.999, 0.5], device=DEV)
     tok, lp, slp = ops.unpack_sample(ops.sample(z, T, u))
