@@ -277,22 +277,24 @@ def test_lookahead_changes_nothing_but_the_timing(tiny_folders, tmp_path):
     assert any(o[-1] in stops and len(o) < p.max_tokens for o, p in zip(outs[True], params)), "no request stopped on an end token"
 
 
-def test_seventy_requests_decode_through_one_graph(tiny_folders):
-    """More rows than the reference's largest captured batch (64): the bucket of 128 rows, with pad rows, against the
-    same run without graphs."""
+@pytest.mark.parametrize("n_requests,bucket", [(70, 96), (100, 128)])
+def test_many_requests_decode_through_one_graph(tiny_folders, n_requests, bucket):
+    """More rows than the reference's largest captured batch (64): the buckets of 96 and 128 rows, with pad rows, against
+    the same run without graphs."""
     from nanospec_amd import SamplingParams
 
     name = "B"
     model = model_of(tiny_folders[name], name, torch.bfloat16)
     vocab = TINY[name]["cfg"]["vocab_size"]
-    prompts = [random_tokens(3 + i % 11, vocab, 900 + i) for i in range(70)]
-    params = [SamplingParams(max_tokens=12 + i % 3) for i in range(70)]
+    prompts = [random_tokens(3 + i % 11, vocab, 900 + i) for i in range(n_requests)]
+    params = [SamplingParams(max_tokens=12 + i % 3) for i in range(n_requests)]
     outs = {}
     for graphs in (True, False):
-        reqs, _, eng = run_engine(model, prompts, params, num_blocks=400, block_size=8, max_admit=70, max_running=70, cuda_graphs=graphs)
+        reqs, _, eng = run_engine(model, prompts, params, num_blocks=600, block_size=8, max_admit=n_requests, max_running=n_requests,
+                                  cuda_graphs=graphs)
         outs[graphs] = [r.out_tokens for r in reqs]
         if graphs:
-            assert 128 in eng.runner._graphs, "the 70 rows did not replay the graph of 128"
+            assert bucket in eng.runner._graphs, f"the {n_requests} rows did not replay the graph of {bucket}"
     assert outs[True] == outs[False]
 
 
