@@ -93,18 +93,23 @@ def decode_run(model, cfg, batch: int, prompt_len: int, first_ctx: int, steps: i
     return dt, ctx0, ctx0 + steps
 
 
-def prefill_run(model, cfg, n_tokens: int, block_size: int, reps: int = 3):
+def prefill_run(model, cfg, n_tokens: int, block_size: int, reps: int = 3, portion: int = 0):
+    """Seconds for a prompt of ``n_tokens``, whole or in portions of ``portion`` tokens (the best of ``reps`` passes)."""
     import torch
 
     from nanospec_amd.engine.replay import Replayer
 
     rep = Replayer(model, n_tokens + 64, page_size=block_size, use_graphs=False)
     toks = torch.randint(0, cfg.vocab_size, (n_tokens,), generator=torch.Generator().manual_seed(7)).tolist()
+    portion = portion or n_tokens
     best = None
     for i in range(reps + 1):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        rep.step([{"id": f"p{i}", "tokens": toks, "want": [n_tokens - 1]}], [f"p{i}"])
+        for s in range(0, n_tokens, portion):
+            last = s + portion >= n_tokens
+            rep.step([{"id": f"p{i}", "tokens": toks[s : s + portion], "want": [min(portion, n_tokens - s) - 1] if last else []}],
+                     [f"p{i}"] if last else [])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         if i and (best is None or dt < best):
@@ -123,6 +128,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true")
+    ap.add_argument("--ctx", type=int, default=2048, help="context of the first timed decode step (the benchmark's is 2,048)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure (the benchmark's is 2,048)")
+    ap.add_argument("--prefill-portion", type=int, default=0, help="take that prompt in portions of this many tokens (0: whole)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -143,18 +151,19 @@ def main() -> int:
     dtype = torch.bfloat16 if a.dtype == "bf16" else torch.float32
     esize = 2 if a.dtype == "bf16" else 4
     model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
-    block, prompt, ctx_end = 16, 2048, 4096
+    block, prompt = 16, 2048
+    ctx_end = a.ctx + a.steps if a.ctx != 2048 else 4096
 
     steps = a.steps
-    dt, ctx0, ctx1 = decode_run(model, cfg, a.batch, prompt, prompt, steps, a.warmup, block, seed=1)
+    dt, ctx0, ctx1 = decode_run(model, cfg, a.batch, prompt, a.ctx, steps, a.warmup, block, seed=1)
     ms = 1000 * dt / steps
     value = a.batch * steps / dt
     mean_ctx = (ctx0 + ctx1 - 1) / 2
     step_bytes = weight_bytes(cfg, esize) + a.batch * mean_ctx * kv_bytes_per_token(cfg, esize)
     achieved = step_bytes / (dt / steps) / 1e9
 
-    p_tokens = 2048
-    p_dt = prefill_run(model, cfg, p_tokens, block)
+    p_tokens = a.prefill_tokens
+    p_dt = prefill_run(model, cfg, p_tokens, block, portion=a.prefill_portion)
     p_frac = prefill_flops(cfg, p_tokens, 1) / p_dt / PEAK_FLOPS[a.dtype]
 
     points = {}
@@ -166,14 +175,14 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * k / d, 1)
 
     line = {
-        "metric": f"decode tok/s at bs {a.batch}, ctx 2048->4096 ({SHAPE_NAMES[a.shape]}, {a.dtype}); prefill tok/s @2048 tok",
+        "metric": f"decode tok/s at bs {a.batch}, ctx {a.ctx}->{ctx_end} ({SHAPE_NAMES[a.shape]}, {a.dtype}); prefill tok/s @{p_tokens} tok",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
         "config": {"model": SHAPE_NAMES[a.shape], "layers": shape["num_hidden_layers"], "layers_of_shape": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": prompt, "ctx_first_step": round(ctx0, 1),
+                   "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": a.ctx, "ctx_first_step": round(ctx0, 1),
                    "ctx_last_step": round(ctx1 - 1, 1), "page_size": block, "parallelism": "single GPU", "graphs": True},
         "prefill": {"value": round(p_tokens / p_dt, 1), "tokens": p_tokens, "ms": round(1000 * p_dt, 3), "frac": round(p_frac, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",

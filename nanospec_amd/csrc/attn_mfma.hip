@@ -473,14 +473,19 @@ constexpr int CPR = PS / 8 < 4 ? PS / 8 : 4;  // 16-byte pieces of a block that 
 
 // Two waves per SIMD: with more registers the compiler parks the sums in accumulation registers and moves them to and
 // fro around every rescaling.
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnParams a) {
+// SETS = 1: one set of four waves per workgroup, which walks all blocks of its range of the tile's keys.  Two such
+// workgroups share a compute unit and each has a barrier of its own, so the two waves of a SIMD are not kept in the same
+// phase and one's matrix instructions run under the other's soft-max arithmetic.  It pays where the ranges are joined by
+// the second kernel anyway or the keys are many (the join costs a pass over the unnormalised sums).
+template <int SETS>
+__global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnParams a) {
   if constexpr (SHARED_OK) {
     constexpr int K_BYTES = 32 * KROW * 2, V_BYTES = HD * VROW * 2, SET_BYTES = 2 * (K_BYTES + V_BYTES);
-    constexpr int JOIN_BYTES = 256 * (2 * DT * 4 + 4) * 4;  // what the second set hands to the first: sums, maxima, totals
-    __shared__ __align__(16) char smem[2 * SET_BYTES > JOIN_BYTES ? 2 * SET_BYTES : JOIN_BYTES];
+    constexpr int JOIN_BYTES = SETS == 2 ? 256 * (2 * DT * 4 + 4) * 4 : 0;  // what the second set hands to the first: sums, maxima, totals
+    __shared__ __align__(16) char smem[SETS * SET_BYTES > JOIN_BYTES ? SETS * SET_BYTES : JOIN_BYTES];
     // What is the same in all lanes of a wave is said to be so (readfirstlane): the loop's branches and the address
     // arithmetic that depends on the block alone then run on the scalar unit, and no branch is taken under a lane mask.
-    const int half = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);  // which set of four waves, i.e. which half of the tile's blocks
+    const int half = SETS == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;  // which set of four waves, i.e. which half of the tile's blocks
     bf16_t(*lk)[32 * KROW] = reinterpret_cast<bf16_t(*)[32 * KROW]>(smem + half * SET_BYTES);
     bf16_t(*lv)[HD * VROW] = reinterpret_cast<bf16_t(*)[HD * VROW]>(smem + half * SET_BYTES + 2 * K_BYTES);
     const int tid = threadIdx.x & 255, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -526,8 +531,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
       tile_kb0 = min(tile_kb1, tile_kb0 + split * per);
       tile_kb1 = min(tile_kb1, tile_kb0 + per);
     }
-    const int steps = (tile_kb1 - tile_kb0 + 1) / 2;  // blocks of the first set; the second has as many or one fewer
-    const int kb0 = half ? tile_kb0 + steps : tile_kb0, kb1 = half ? tile_kb1 : tile_kb0 + steps;
+    const int steps = SETS == 2 ? (tile_kb1 - tile_kb0 + 1) / 2 : tile_kb1 - tile_kb0;  // blocks of the first set; the second has as many or one fewer
+    const int kb0 = half ? tile_kb0 + steps : tile_kb0, kb1 = (half || SETS == 1) ? tile_kb1 : tile_kb0 + steps;
 
     bf16x8 qw[2][NQ];
 #pragma unroll
@@ -744,7 +749,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
     // The second set hands its sums to the first, lane by lane (both hold the same columns and channels):
     // o = o_0 2^((m_0 - m*) scale) + o_1 2^((m_1 - m*) scale), likewise the totals, m* = max(m_0, m_1).
     float* join = reinterpret_cast<float*>(smem) + tid * (2 * DT * 4 + 4);
-    if (half) {
+    if (SETS == 2 && half) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
 #pragma unroll
@@ -753,10 +758,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void a
         join[2 * DT * 4 + 2 + u] = lsum[u];
       }
     }
-    __syncthreads();
+    if (SETS == 2) __syncthreads();
     if (half) return;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; SETS == 2 && u < 2; ++u) {
       const float m1 = join[2 * DT * 4 + u], l1 = join[2 * DT * 4 + 2 + u];
       const float mstar = fmaxf(m[u], m1);
       const float msafe = mstar == -INFINITY ? 0.f : mstar;
@@ -870,7 +875,8 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (hp != 1 && hp != 2 && hp != 4 && hp != 8 && hp != 16) return NS_ERR_BAD_ARG;
   if (!(scale > 0.f)) return NS_ERR_BAD_ARG;  // maxima are tracked on unscaled scores
   if (splits > 1 && (!part_o || !part_ml)) return NS_ERR_BAD_ARG;
-  if (qt != 1 && !(qt == 2 && hp == 1 && !coop)) return NS_ERR_BAD_ARG;
+  // (with qt == 2, coop asks for one set of four waves per workgroup: see attn_prefill_kernel)
+  if (qt != 1 && !(qt == 2 && hp == 1)) return NS_ERR_BAD_ARG;
   AttnParams a;
   a.out = (bf16_t*)out; a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
   a.q = (const bf16_t*)q; a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
@@ -885,7 +891,10 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (qt == 2 && SHARED_OK) {
     const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
-    attn_prefill_kernel<<<(unsigned)wgs, 512, 0, stream>>>(a);
+    if (coop)
+      attn_prefill_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>(a);
+    else
+      attn_prefill_kernel<2><<<(unsigned)wgs, 512, 0, stream>>>(a);
   } else if (qt == 2)
     attn_mfma_kernel<2, false, false><<<(unsigned)blocks, 256, 0, stream>>>(a);
   else if (coop)

@@ -26,6 +26,7 @@ import torch
 
 CHUNK_TILE = 32  # tokens per attention tile of a prompt portion (two 16-column tiles per wave)
 CHUNK_RANGE_BLOCKS = 16  # the fewest 32-key blocks that a range of a prompt portion's keys is worth a workgroup of its own
+CHUNK_SINGLE_SET_BLOCKS = 128  # 32-key blocks of the longest row from which a workgroup is one set of waves instead of two
 CHUNK_FILL = 256  # workgroups of prompt-portion tiles (one fits a compute unit) below which their keys are cut into ranges
 TILE_INTS = 8  # a tile descriptor: request, first token, row of the request's first token, tokens, keys, 0, 0, 0
 
@@ -106,7 +107,10 @@ class StepContext:
             if splits > 1:
                 cols = lay.Tc * CHUNK_TILE * kv_heads * group
                 ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
-            plans.append(AttentionPlan(self._ctiles, 1, splits, ws, qt=CHUNK_TILE // 16))
+            # many workgroups with long rows of keys: one set of four waves per workgroup, two workgroups to a compute unit,
+            # each with a barrier of its own (4 to 8% faster from 4,096 keys on; slower for short rows)
+            single = splits == 1 and wgs >= 2 * CHUNK_FILL and blocks >= CHUNK_SINGLE_SET_BLOCKS
+            plans.append(AttentionPlan(self._ctiles, 1, splits, ws, qt=CHUNK_TILE // 16, coop=single))
         if lay.Td:
             hp = 1
             while hp < min(group, 16):

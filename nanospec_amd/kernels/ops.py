@@ -550,7 +550,8 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     request in this step, keys after this step, three zeros).  ``hp`` heads of a group times 16/hp tokens make a tile;
     with ``qt`` = 2 (only with hp = 1) a tile is 32 tokens.  ``splits`` > 1 cuts the keys of every tile
     into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors.  With ``coop`` the four
-    waves of a workgroup share each tile and range (for decode, where a wave's chain of loads is what takes the time)."""
+    waves of a workgroup share each tile and range (for decode, where a wave's chain of loads is what takes the time); with
+    ``qt`` = 2 it asks for workgroups of one set of four waves instead of two (for long rows of keys)."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
     if not mfma_attention_takes(q.dtype, head_dim, page):
         raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
@@ -561,8 +562,8 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
         raise KernelRefused(f"attention_mfma: tiles must be int32 [n_tiles, {TILE_INTS}], 16-byte aligned")
     if hp not in (1, 2, 4, 8, 16):
         raise KernelRefused("attention_mfma: hp is a power of two up to 16")
-    if qt != 1 and not (qt == 2 and hp == 1 and not coop):
-        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1 and no cooperating waves")
+    if qt != 1 and not (qt == 2 and hp == 1):
+        raise KernelRefused("attention_mfma: 32-token tiles (qt = 2) go with hp = 1")
     n_tiles = tiles.shape[0]
     po = pm = None
     if splits > 1:

@@ -510,7 +510,7 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
         if chunk_splits > 1:  # filled with NaN: a range that is read without having been written shows
             ws = (torch.full((cols * chunk_splits * hd,), float("nan"), device=DEV), torch.full((cols * chunk_splits * 2,), float("nan"), device=DEV))
         ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1,
-                           splits=chunk_splits, workspace=ws, qt=qt)
+                           splits=chunk_splits, workspace=ws, qt=qt, coop=coop and qt == 2)  # coop: one set of waves per workgroup
     if dt:
         hp = 1
         while hp < min(group, 16):
@@ -541,7 +541,7 @@ def test_attention_mfma(case, heads, kvh, hd, page):
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
     # the last number: ranges that the keys of a prompt portion's tiles are cut into (16: more than most tiles have blocks)
     for splits, qt, coop, step_keys, chunk_splits in ((1, 2, False, 0, 1), (3, 1, False, 0, 2), (7, 2, True, 0, 3), (33, 1, False, 2**30, 1),
-                                                      (1, 1, True, 2**30, 5), (2, 2, True, 0, 16)):
+                                                      (1, 1, True, 2**30, 5), (2, 2, True, 0, 16), (1, 2, True, 0, 1)):
         out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, force_splits=splits, qt=qt, coop=coop, step_keys=step_keys,
                         chunk_splits=chunk_splits)
         u = ulps_of_row_max(out.cpu(), ref).max()
@@ -599,6 +599,8 @@ def test_attention_window(kernel, window):
     if kernel == "mfma":
         out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=window)
         cut = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=window, chunk_splits=3)
+        assert ulps_of_row_max(cut.cpu(), ref).max() <= 4
+        cut = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=window, chunk_splits=2, coop=True)
         assert ulps_of_row_max(cut.cpu(), ref).max() <= 4
     else:
         positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
