@@ -321,8 +321,8 @@ def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight 
         raise KernelRefused("linear_tiled: w2 must match w")
     if waves == 0:  # with more than 8 rows eight waves were never behind four at the shapes measured
         waves = 8 if w.k >= 8192 or ((w.n // 16 < 512 or m > 8) and w.k >= 2048) else 4
-    if halves is None:
-        halves = m <= GATED_HALF_ROWS
+    if halves is None:  # (with 3 or 4 rows only where whole row tiles would not spread evenly over 256 compute units)
+        halves = m <= 2 or (m <= GATED_HALF_ROWS and -(-w.n // 16) % 256 != 0)
     epi = 0 if w2 is None else (4 if halves and m <= 16 and not out_f32 else 1)
     _check(build.core().ns_gemm_tiled_bf16(_ptr(out), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None), c_int(m),
                                            c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
