@@ -277,7 +277,7 @@ def test_lookahead_changes_nothing_but_the_timing(tiny_folders, tmp_path):
     assert any(o[-1] in stops and len(o) < p.max_tokens for o, p in zip(outs[True], params)), "no request stopped on an end token"
 
 
-@pytest.mark.parametrize("n_requests,bucket", [(70, 96), (100, 128)])
+@pytest.mark.parametrize("n_requests,bucket", [(40, 48), (70, 96), (100, 128)])
 def test_many_requests_decode_through_one_graph(tiny_folders, n_requests, bucket):
     """More rows than the reference's largest captured batch (64): the buckets of 96 and 128 rows, with pad rows, against
     the same run without graphs."""
