@@ -24,8 +24,10 @@ from .arena import Arena
 from .context import BatchLayout, StepContext, count_tiles, fill_batch
 
 # reference: engine/graphs.py:22 (powers of two up to 64).  48 and 96 besides: the products' cost goes by 16 rows at a time
-# between 17 and 128 rows, so 40 requests padded to 64 rows pay for a quarter more than padded to 48.
-GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 256)
+# between 17 and 128 rows, so 40 requests padded to 64 rows pay for a quarter more than padded to 48.  Above 128 rows
+# the library's products take the steps; 176, 208 and 240 are row counts at which its choice of kernels was measured to
+# be good for all four shapes of a layer (160, 192 and 256 are not: q/k/v takes 40 us at 256 rows and 27 at 240).
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 176, 208, 240, 256)
 PAD_REQUEST = "__pad__"
 
 
