@@ -1,9 +1,10 @@
-// bfloat16 matrix products on the matrix cores for 17 to 64 rows, and for up to 128 rows of one matrix with one row tile
-// per wave (decode at large batch, short portions):
+// bfloat16 matrix products on the matrix cores for 17 to 64 rows, for up to 128 rows of one matrix with one row tile per
+// wave (decode at large batch, short portions), and for any number of rows in blocks of 128 with two or four row tiles per
+// wave (ns_gemm_rows_bf16: the prompts of models that keep the tiled layout only):
 //   out[M, N] = x[M, K] . w[N, K]^T,  32-bit accumulation, weights in the tiled layout of gemm_bf16.hip.
 //
 // With this many rows the traffic of x counts: a workgroup of 4 waves owns 64 rows of w (16 per wave) and all its
-// waves walk through the same k tiles, so that a tile of x (64 tokens x 128 k) is fetched once per workgroup, with
+// waves walk through the same k tiles, so that a tile of x (up to 128 tokens x 128 k) is fetched once per workgroup, with
 // whole-row loads, into LDS and read from there by every wave in the layout the matrix instruction wants.  The weights
 // still go from memory straight into registers, each exactly once.  Since 64 rows per workgroup leave too few workgroups
 // to fill the GPU, K is cut into `ksplit` ranges over blockIdx.y; each range writes 32-bit partial sums and a second
