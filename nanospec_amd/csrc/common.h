@@ -13,6 +13,7 @@ typedef __bf16 bf16_t;
 #define NS_OK 0
 #define NS_ERR_BAD_ARG 1001
 #define NS_ERR_UNSUPPORTED 1002
+#define NS_ERR_SCRATCH_TOO_SMALL 1003
 
 template <typename T> __device__ __forceinline__ float to_f(T v) { return (float)v; }
 template <typename T> __device__ __forceinline__ T from_f(float v) { return (T)v; }

@@ -12,6 +12,7 @@
 // single range the first kernel applies the epilogue itself and nothing is written twice.
 // (reference for the products: the nn.Linear calls of model/llama.py:175,184,195,286)
 #include "common.h"
+#include "no_alloc.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
@@ -241,9 +242,8 @@ static int launch_wide_tall(float* partial, const bf16_t* x, const bf16_t* wt, i
 // workspace: (wt2 ? 2 : 1) * ksplit * M * N floats (unused with ksplit == 1).  epi 0: store; 1: silu(x.w^T) * (x.w2^T).
 // defer (with ksplit > 1 and epi 0): the ranges stay in the workspace as [ksplit][M][N] and nothing is written to out; they
 // are added later by ns_wide_reduce or by a norm that reads them (ns_rmsnorm_partial).
-extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
-                                 int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer,
-                                 hipStream_t stream) {
+static int wide_product(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N, int K,
+                        int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer, hipStream_t stream) {
   if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
   if (M > 64 && (wt2 != nullptr || nt != 1)) return NS_ERR_BAD_ARG;  // 65 to 128 rows: one matrix, one row tile per wave
   if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
@@ -274,6 +274,56 @@ extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, cons
   else
     gemm_wide_reduce_kernel<bf16_t, 0><<<blocks, 256, 0, stream>>>((bf16_t*)out, part, M, N, out_stride, ksplit);
   return ns_launch_status();
+}
+
+extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
+                                 int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer,
+                                 hipStream_t stream) {
+  return wide_product(out, workspace, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, ksplit, nt, defer, stream);
+}
+
+// ------------------------------------------------------------------ the same product without a workspace argument
+// The partial sums of the ranges lie in an array of the library's own (see no_alloc.h).  In host code the array's name is
+// only a handle for hipGetSymbolAddress: every GPU has its own copy at its own address, which is looked up once per GPU,
+// with that GPU current, and kept; only that address is ever given to a kernel.
+static __device__ __align__(256) float scratch[NS_STATIC_SCRATCH_FLOATS];
+
+#define NS_MAX_GPUS 64
+static float* scratch_ptr[NS_MAX_GPUS];  // per GPU: the address of its copy of `scratch`, nullptr until looked up
+
+// -> this GPU's copy of the array, or nullptr with *err set.
+static float* static_scratch(int* err) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { *err = (int)e; return nullptr; }
+  if (dev < 0 || dev >= NS_MAX_GPUS) { *err = NS_ERR_BAD_ARG; return nullptr; }
+  float* p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p) return p;
+  void* found = nullptr;
+  e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !found) { *err = e != hipSuccess ? (int)e : NS_ERR_UNSUPPORTED; return nullptr; }
+  __atomic_store_n(&scratch_ptr[dev], (float*)found, __ATOMIC_RELEASE);  // two threads at once find the same address
+  return (float*)found;
+}
+
+extern "C" int ns_static_scratch_init(void) {
+  int err = NS_OK;
+  return static_scratch(&err) ? NS_OK : err;
+}
+
+extern "C" int ns_gemm_wide_bf16_static(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
+                                        int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt,
+                                        hipStream_t stream) {
+  if (M <= 0 || N <= 0 || ksplit < 1 || !out) return NS_ERR_BAD_ARG;
+  float* ws = nullptr;
+  if (ksplit > 1) {
+    const unsigned long long need = (unsigned long long)(wt2 ? 2 : 1) * (unsigned long long)ksplit * (unsigned long long)M * (unsigned long long)N;
+    if (need > NS_STATIC_SCRATCH_FLOATS) return NS_ERR_SCRATCH_TOO_SMALL;
+    int err = NS_OK;
+    ws = static_scratch(&err);
+    if (!ws) return err;
+  }
+  return wide_product(out, ws, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, ksplit, nt, 0, stream);
 }
 
 // Any number of rows, 128 at a time over blockIdx.z, with `nt` row tiles of w per wave (2 or 4; 1 or 2 with wt2): each

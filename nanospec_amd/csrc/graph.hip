@@ -28,5 +28,6 @@ extern "C" int ns_graph_destroy(void* exec) { return (int)hipGraphExecDestroy((h
 extern "C" const char* ns_error_string(int code) {
   if (code == NS_ERR_BAD_ARG) return "bad argument (a size the kernel does not take)";
   if (code == NS_ERR_UNSUPPORTED) return "unsupported dtype or option";
+  if (code == NS_ERR_SCRATCH_TOO_SMALL) return "the product needs more partial sums than the library's own array holds";
   return hipGetErrorString((hipError_t)code);
 }

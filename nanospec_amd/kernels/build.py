@@ -56,7 +56,7 @@ def _hipcc() -> str:
 
 def _digest(sources: list[str], defines: list[str]) -> str:
     h = hashlib.sha256()
-    for name in sorted(set(sources) | {"common.h"}):
+    for name in sorted(set(sources) | {h.name for h in CSRC.glob("*.h")}):
         h.update(name.encode())
         h.update((CSRC / name).read_bytes())
     h.update(" ".join(FLAGS + defines).encode())
