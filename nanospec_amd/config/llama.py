@@ -140,7 +140,9 @@ class LlamaConfig:
                              head_dim=self.head_dim, position=rope, softmax_scale=1.0 / math.sqrt(self.head_dim))
         ffn = SwiGLUSpec(hidden=self.hidden_size, intermediate=self.intermediate_size)
         layers = tuple(
-            PreNormBlockSpec(prefix=f"model.layers.{i}.", mixer_norm=norm, mixer=attn, ffn_norm=norm, ffn=ffn)
+            PreNormBlockSpec(prefix=f"model.layers.{i}.", mixer_norm=norm, mixer=attn, ffn_norm=norm, ffn=ffn,
+                             mixer_norm_name="input_layernorm.weight", mixer_prefix="self_attn.",
+                             ffn_norm_name="post_attention_layernorm.weight", ffn_prefix="mlp.")
             for i in range(self.num_hidden_layers)
         )
         return ModelSpec(

@@ -69,7 +69,9 @@ class SwiGLUSpec:
 @dataclass(frozen=True)
 class PreNormBlockSpec:
     """x = x + mixer(norm1(x)); x = x + feed_forward(norm2(x)).  ``prefix`` is the layer's
-    tensor-name prefix in the checkpoint, e.g. ``model.layers.3.``."""
+    tensor-name prefix in the checkpoint, e.g. ``model.layers.3.``; the four names that follow it are the
+    architecture's own and are appended to it: the two norms' weight tensors and the prefixes under which
+    the mixer and the feed-forward find their tensors (None: the part's ``kind`` and a dot)."""
 
     kind: ClassVar[str] = "prenorm"
     prefix: str
@@ -77,6 +79,10 @@ class PreNormBlockSpec:
     mixer: object
     ffn_norm: object
     ffn: object
+    mixer_norm_name: str = "mixer_norm.weight"
+    mixer_prefix: str | None = None
+    ffn_norm_name: str = "ffn_norm.weight"
+    ffn_prefix: str | None = None
 
 
 @dataclass(frozen=True)

@@ -19,15 +19,10 @@ Slots are not materialised: the kernels compute page and offset from the positio
 
 from __future__ import annotations
 
-from dataclasses import dataclass
-
 import numpy as np
 import torch
 
-CHUNK_TILE = 32  # tokens per attention tile of a prompt portion (two 16-column tiles per wave)
-CHUNK_RANGE_BLOCKS = 16  # the fewest 32-key blocks that a range of a prompt portion's keys is worth a workgroup of its own
-CHUNK_SINGLE_SET_BLOCKS = 128  # 32-key blocks of the longest row from which a workgroup is one set of waves instead of two
-CHUNK_FILL = 256  # workgroups of prompt-portion tiles (one fits a compute unit) below which their keys are cut into ranges
+CHUNK_TILE = 32  # tokens per tile of a prompt portion in the batch's tile lists
 TILE_INTS = 8  # a tile descriptor: request, first token, row of the request's first token, tokens, keys, 0, 0, 0
 
 
@@ -56,20 +51,10 @@ class BatchLayout:
         self.total = off
 
 
-@dataclass
-class AttentionPlan:
-    tiles: torch.Tensor  # int32 [n_tiles, 8]
-    hp: int
-    splits: int
-    workspace: tuple | None
-    qt: int = 1
-    coop: bool = False
-
-
 class StepContext:
     """Device views of one step's batch plus the arena; handed to every part."""
 
-    def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, fixed_splits: bool = False,
+    def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, captured: bool = False,
                  link_norms: bool = True, max_chunk_kv: int | None = None) -> None:
         self.layout, self.arena = layout, arena
         # the most keys that a request bringing a prompt portion has after this step (at most max_kv_len)
@@ -78,7 +63,9 @@ class StepContext:
         self.link_norms = link_norms
         self.n_tokens, self.n_reqs = layout.N, layout.B
         self.max_position, self.max_kv_len = max_position, max_kv_len
-        self.fixed_splits = fixed_splits
+        # the step is being captured for replays with other lengths (up to max_kv_len keys): a part's choices may depend
+        # on the counts of the batch but not on this step's lengths
+        self.captured = captured
         f = layout.fields
 
         def view(name):
@@ -88,48 +75,13 @@ class StepContext:
         self.token_ids, self.positions, self.token_req = view("token_ids"), view("positions"), view("token_req")
         self.qo_indptr, self.kv_lens, self.state_slots = view("qo_indptr"), view("kv_lens"), view("state_slots")
         self.want_rows = view("want_rows")
-        self._ctiles = view("ctiles").view(-1, TILE_INTS)
-        self._dtiles = view("dtiles").view(-1, TILE_INTS)
+        # The requests of the batch as tiles, for mixers that work tile by tile: those that bring more than one token cut
+        # into tiles of CHUNK_TILE tokens, and those that bring exactly one (int32 [tiles, TILE_INTS] each, see above)
+        self.chunk_tiles = view("ctiles").view(-1, TILE_INTS)
+        self.decode_tiles = view("dtiles").view(-1, TILE_INTS)
+        self.n_chunk_tiles, self.n_decode_tiles = layout.Tc, layout.Td
+        self.chunk_tiles_tokens = CHUNK_TILE
         self.block_tables = [dev_buf[o : o + layout.B * layout.P].view(layout.B, layout.P) for o in layout.table_off]
-
-    def attention_plans(self, group: int, kv_heads: int, head_dim: int) -> list[AttentionPlan]:
-        """How the matrix-core attention kernel is launched for a mixer with ``group`` query heads per
-        key/value head: prompt portions as 32-token tiles of one head, their keys cut into ranges when there are too few
-        tiles to fill the GPU and many keys (a short portion late in a long prompt); decode rows with all heads of a
-        group in one tile and the keys cut into ranges so that the launch fills the GPU."""
-        plans = []  # made afresh per call: the workspace lives in the caller's arena scope
-        lay = self.layout
-        if lay.Tc:
-            wgs = lay.Tc * kv_heads * -(-group // 4)
-            blocks = -(-self.max_chunk_kv // 32)
-            splits = max(1, min(16, CHUNK_FILL // wgs, blocks // CHUNK_RANGE_BLOCKS))
-            ws = None
-            if splits > 1:
-                cols = lay.Tc * CHUNK_TILE * kv_heads * group
-                ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
-            # many workgroups with long rows of keys: one set of four waves per workgroup, two workgroups to a compute unit,
-            # each with a barrier of its own (4 to 8% faster from 4,096 keys on; slower for short rows)
-            single = splits == 1 and wgs >= 2 * CHUNK_FILL and blocks >= CHUNK_SINGLE_SET_BLOCKS
-            plans.append(AttentionPlan(self._ctiles, 1, splits, ws, qt=CHUNK_TILE // 16, coop=single))
-        if lay.Td:
-            hp = 1
-            while hp < min(group, 16):
-                hp *= 2
-            # decode is bound by the latency of each wave's chain of loads: the four waves of a workgroup share a tile, and
-            # the keys are cut into ranges until about a thousand waves are at work
-            # (up to 32 ranges where requests may reach 8,192 keys and the tiles are few, a single request say: at 131,072
-            # keys 86 against 132 us a layer; the kernel leaves the ranges beyond the sixteenth empty for shorter rows,
-            # and where no request can be that long they are not launched: they would cost a captured step 1%)
-            items = lay.Td * kv_heads * -(-group // hp)
-            splits = max(1, min(32 if self.max_kv_len >= 8192 else 16, 1024 // (4 * items)))
-            if not self.fixed_splits:
-                splits = max(1, min(splits, -(-self.max_kv_len // 256)))
-            ws = None
-            if splits > 1:
-                cols = lay.Td * (16 // hp) * kv_heads * group
-                ws = (self.arena.take((cols * splits * head_dim,), torch.float32), self.arena.take((cols * splits * 2,), torch.float32))
-            plans.append(AttentionPlan(self._dtiles, hp, splits, ws, coop=True))
-        return plans
 
 
 def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, slots, want_rows, tables: list[np.ndarray],

@@ -33,7 +33,7 @@ class EngineConfig:
     max_step_tokens: int | None = None  # token budget of a step; None = whole prompts, as the reference
     prefill_chunk: int | None = None  # longest portion of one prompt in a step
     on_exhaustion: str = "reserve"  # "reserve" | "preempt": see engine/scheduler.py
-    max_seq_len: int | None = None  # longest request (sizes the block tables); None = the whole pool
+    max_seq_len: int | None = None  # longest request that is accepted; None = what the model's positions and the pool allow
     lookahead: bool = True  # enqueue the next decode step before waiting for this one's tokens
 
 
@@ -48,7 +48,12 @@ class Engine:
         num_slots = max_running + 1  # one for the pad rows of captured graphs
         self.cache = CacheManager(specs, config.num_blocks, config.block_size, num_slots)
         self.storage = CacheStorage(model, [config.num_blocks] * len(specs), config.block_size, num_slots, self.dtype, self.device)
-        width = config.num_blocks if config.max_seq_len is None else -(-config.max_seq_len // config.block_size)
+        # the longest request: what the caller says and the model's positions allow (the pool bounds it too; the scheduler
+        # refuses what can never fit it).  Block tables are only ever as wide as the live requests need: the runner's
+        # captured steps grow with them.
+        limits = [n for n in (model.max_positions, config.max_seq_len) if n is not None]
+        self.max_seq_len = min(limits) if limits else None
+        width = config.num_blocks if self.max_seq_len is None else min(config.num_blocks, -(-self.max_seq_len // config.block_size))
         self.runner = ModelRunner(model, self.cache, self.storage, max_running, width, use_graphs=config.cuda_graphs)
         self.sched = Scheduler(self.cache, config.max_admit, config.max_running, config.max_step_tokens, config.prefill_chunk,
                                config.on_exhaustion)
@@ -88,6 +93,10 @@ class Engine:
         vocab = self.model.spec.vocab_size
         if any(not 0 <= int(t) < vocab for t in prompt_ids):
             raise ValueError(f"prompt holds a token id outside [0, {vocab})")
+        if self.max_seq_len is not None and len(prompt_ids) + params.max_tokens - 1 > self.max_seq_len:
+            # (the last sampled token is never fed back, so a request holds at most prompt + max_tokens - 1 positions)
+            raise ValueError(f"a prompt of {len(prompt_ids)} tokens with max_tokens={params.max_tokens} runs past the "
+                             f"{self.max_seq_len} positions that the model and the engine's settings allow")
         req = Request(self._next_id, [int(t) for t in prompt_ids], params)
         self._next_id += 1
         self.sched.add(req)
@@ -121,7 +130,11 @@ class Engine:
                     return []
                 launched = self._launch(work, None)
             if self._may_look_ahead(launched):
-                self._ahead = self._launch_ahead(launched)
+                try:
+                    self._ahead = self._launch_ahead(launched)
+                except Exception:
+                    self._harvest(launched)  # this step's tokens are not lost to a failure of the next one's launch
+                    raise
             return self._harvest(launched)
 
     def _launch(self, work: list[Work], token_src) -> dict:

@@ -21,12 +21,12 @@ MAX_LIVE = 4  # requests a trace keeps alive at a time; one more slot serves the
 
 
 class Replayer:
-    def __init__(self, model, max_tokens: int, page_size: int = 16, use_graphs: bool = True) -> None:
+    def __init__(self, model, max_tokens: int, page_size: int = 16, use_graphs: bool = True, max_live: int = MAX_LIVE) -> None:
         self.model = model
         specs, _, _ = plan_groups(model.cache_needs)
         # room for ``max_tokens`` tokens of live requests, each rounded up to whole pages, plus the pad page
         pages = -(-max_tokens // page_size) + 1
-        slots = MAX_LIVE + 4
+        slots = max_live + 4
         self.manager = CacheManager(specs, pages, page_size, slots)
         self.storage = CacheStorage(model, [pages] * len(specs), page_size, slots, model.dtype, model.device)
         self.runner = ModelRunner(model, self.manager, self.storage, slots, pages, use_graphs=use_graphs)

@@ -42,10 +42,10 @@ class _DecodeGraph:
     """One captured decode step for a bucket of ``size`` requests: static batch buffer, fixed arena,
     logits for every row."""
 
-    def __init__(self, runner: "ModelRunner", size: int) -> None:
-        self.size = size
+    def __init__(self, runner: "ModelRunner", size: int, width: int) -> None:
+        self.size, self.width = size, width  # rows; pages per request that its block tables can name
         n_groups = len(runner.manager.groups)
-        self.layout = BatchLayout(size, size, size, 0, size, n_groups, runner.table_width, n_patch=size, n_sample=size)
+        self.layout = BatchLayout(size, size, size, 0, size, n_groups, width, n_patch=size, n_sample=size)
         dev = runner.device
         self.dev_buf = torch.zeros(self.layout.total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
@@ -63,8 +63,8 @@ class _DecodeGraph:
         return f[0], f[1], f[2], opts[3]
 
     def context(self, runner) -> StepContext:
-        return StepContext(self.layout, self.dev_buf, self.arena, link_norms=runner.link_norms, max_position=0, max_kv_len=runner.table_width * runner.page_size,
-                           fixed_splits=True)
+        return StepContext(self.layout, self.dev_buf, self.arena, link_norms=runner.link_norms, max_position=0,
+                           max_kv_len=self.width * runner.page_size, captured=True)
 
 
 class ModelRunner:
@@ -73,9 +73,12 @@ class ModelRunner:
         self.model, self.manager, self.storage = model, manager, storage
         self.device, self.dtype = model.device, model.dtype
         self.page_size = manager.page_size
-        self.table_width = table_width  # pages per request a block table can name
+        self.table_width = table_width  # the most pages that a request's block table can name
         self.max_requests = max_requests
         self.stream = torch.cuda.Stream(device=self.device)
+        # whatever the caller's stream still has to do to the weights and the cache (copies, the pools' zero fill) comes
+        # before the first step on this one
+        self.stream.wait_stream(torch.cuda.current_stream(self.device))
         self.arena = Arena(self.device)
         self._kv_layers = sum(1 for need in model.cache_needs if need is not None and hasattr(need, "kv_heads"))
         self.link_norms = True  # see StepContext; set False before the first step to run every norm as a kernel of its own
@@ -87,7 +90,7 @@ class ModelRunner:
         self._host = torch.zeros(1 << 14, dtype=torch.int32).pin_memory()
         self._dev = torch.zeros(1 << 14, dtype=torch.int32, device=self.device)
         self.use_graphs = bool(use_graphs and model.graph_safe)
-        self._graphs: dict[int, _DecodeGraph] = {}
+        self._graphs: dict[int, _DecodeGraph] = {}  # by rows; one per bucket, recaptured wider when a request outgrows it
         self._pad_ready = False
         self._staged: torch.cuda.Event | None = None
         self.last_used_graph = False
@@ -211,6 +214,7 @@ class ModelRunner:
         n_tokens = sum(lens)
         tc, td = count_tiles(lens)
         max_kv = max(s + n for s, n in zip(starts, lens))
+        self.model.check_positions(max_kv - 1)
         width = max(1, -(-max_kv // self.page_size))
         n_patch = len(device_tokens[1]) if device_tokens else 0
         layout = BatchLayout(n_tokens, len(entries), n_want, tc, td, len(self._tables), width, n_patch)
@@ -263,7 +267,7 @@ class ModelRunner:
         slots = [rc.slot for rc in rcs] + [pad.slot] * n_pad
         token_ids = [e.tokens[0] for e in entries] + [0] * n_pad
         st = list(starts) + [0] * n_pad
-        tables = [t[slots, :] for t in self._tables]
+        tables = [t[slots, : g.width] for t in self._tables]
         fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables, self._kv_layers)
         if device_tokens:
             self._put_patch(g.host_np, g.layout, [e for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
@@ -286,8 +290,24 @@ class ModelRunner:
         if device_tokens:
             self._apply_patch(g.dev_buf, g.layout, device_tokens[0], len(device_tokens[1]))
 
-    def _capture(self, size: int) -> _DecodeGraph:
-        g = _DecodeGraph(self, size)
+    GRAPH_MIN_WIDTH = 16  # pages per request that the narrowest captured step's block tables hold
+
+    def _graph_for(self, size: int, pages: int) -> _DecodeGraph:
+        """The captured step of ``size`` rows, its block tables wide enough for ``pages`` pages per request.  Tables are as
+        wide as the longest request has needed so far, rounded up to a power of two (every replay fills and copies rows x
+        width ints), so a bucket is captured again, twice as wide, when a request outgrows it."""
+        g = self._graphs.get(size)
+        if g is not None and g.width >= pages:
+            return g
+        width = max(self.GRAPH_MIN_WIDTH, 1 << (pages - 1).bit_length())
+        width = min(width, self.table_width)
+        if g is not None:
+            self.stream.synchronize()  # the narrower graph may still be running
+            del self._graphs[size]
+        return self._capture(size, width)
+
+    def _capture(self, size: int, width: int) -> _DecodeGraph:
+        g = _DecodeGraph(self, size, width)
         self._fill_graph(g, [], [], [])
         ctx = g.context(self)
 
@@ -313,11 +333,12 @@ class ModelRunner:
     def _step_graph(self, entries, rcs, starts, device_tokens=None, sampling=None):
         self._ensure_pad()
         size = self._bucket(len(entries))
-        g = self._graphs.get(size) or self._capture(size)
         max_kv = max(starts) + 1
-        if -(-max_kv // self.page_size) > self.table_width:
-            raise ValueError("a request is longer than the block tables of the captured graphs")
-        self._check_positions(max_kv - 1)
+        pages = -(-max_kv // self.page_size)
+        if pages > self.table_width:
+            raise ValueError(f"a request needs {pages} pages; block tables hold {self.table_width}")
+        self.model.check_positions(max_kv - 1)
+        g = self._graph_for(size, pages)
         self._fill_graph(g, entries, rcs, starts, device_tokens, sampling)
         g.graph.launch()
         if sampling is not None and all(e.want for e in entries):
@@ -326,12 +347,6 @@ class ModelRunner:
         if len(rows) == len(entries):
             return g.logits[: len(entries)]
         return g.logits[rows]
-
-    def _check_positions(self, max_position: int) -> None:
-        for layer in self.model.layers:
-            limit = getattr(getattr(layer.mixer, "position", None), "max_positions", None)
-            if limit is not None and max_position >= limit:
-                raise ValueError(f"position {max_position} is beyond the model's {limit} positions")
 
     def synchronize(self) -> None:
         self.stream.synchronize()

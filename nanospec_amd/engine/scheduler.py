@@ -12,6 +12,9 @@ still to be computed.  It samples in the step that consumes its last known token
 
 Token budget (``max_step_tokens``): decoding requests come first with one token each; what is left is
 given to unfinished prompts in admission order, at most ``prefill_chunk`` tokens per request and step.
+When the budget does not even cover the decoding requests, those that have waited longest since their
+last step go first (so that all of them advance in turn), and an eighth of the budget (at least one
+token) is kept for the oldest unfinished prompt, so that it advances too.
 
 Pages running out, by ``on_exhaustion``:
   "reserve"  (default, the reference's way): cannot happen; admission waits until the worst case fits.
@@ -46,6 +49,7 @@ class Request:
     logprobs: list[TokenInfo] = field(default_factory=list)  # only with params.logprobs
     step_logits: list = field(default_factory=list)  # only with EngineConfig.record_logits
     preemptions: int = 0
+    served_at: int = -1  # the scheduler's ticket for this request's last step: smaller = longer ago
 
     def __post_init__(self) -> None:
         if not self.prompt_ids:
@@ -96,6 +100,7 @@ class Scheduler:
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []
         self.preempted_total = 0
+        self.batches = 0  # tickets given so far (one per request and step)
         # hooks the engine sets so that device state follows admission and release
         self.on_admit = cache.admit
         self.on_release = cache.release
@@ -164,6 +169,10 @@ class Scheduler:
             work = self._compose()
             short = self._pages_short(work)
             if not short:
+                # tickets in the order of the last ones: who was served earliest then is earliest again (a round robin)
+                for w in sorted(work, key=lambda w: w.req.served_at):
+                    self.batches += 1
+                    w.req.served_at = self.batches
                 return work
             if self.on_exhaustion != "preempt":
                 raise PoolExhausted("pages ran out although admission reserves the worst case")
@@ -176,6 +185,10 @@ class Scheduler:
         work: list[Work] = []
         decoding = [r for r in self.running if r.seq_len - r.computed == 1]
         filling = [r for r in self.running if r.seq_len - r.computed > 1]
+        if budget is not None and len(decoding) + (1 if filling else 0) > budget:
+            # not every decoding request fits: the longest-waiting first, and a share for the oldest unfinished prompt
+            share = max(1, budget // 8) if filling and budget > 1 else 0
+            decoding = sorted(decoding, key=lambda r: r.served_at)[: budget - share]
         for r in decoding:
             if budget is not None and budget <= 0:
                 break

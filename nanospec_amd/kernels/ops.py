@@ -58,6 +58,19 @@ def _check(code: int, what: str) -> None:
         raise KernelRefused(f"{what}: {msg} (code {code})")
 
 
+_units: dict[int, int] = {}
+
+
+def compute_units(device) -> int:
+    """Compute units of the GPU a tensor lives on (256 on an MI355X); launch heuristics count workgroups against it."""
+    index = torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index not in _units:
+        _units[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return _units[index]
+
+
 def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
     if t.dtype != torch.int32 or not t.is_contiguous():
         raise KernelRefused(f"{name} must be a contiguous int32 tensor")

@@ -10,17 +10,78 @@ all heads of a group with the keys cut into ranges that are joined afterwards.
 
 from __future__ import annotations
 
+from dataclasses import dataclass
+
 import torch
 
 from ..kernels import ops
 from . import registry
-from .linear import Layouts, LinearWeight
+from .linear import LinearWeight
 from .needs import PagedNeed
+
+# How the matrix-core attention kernel is launched, from the counts of a step's batch and the size of the GPU
+PORTION_RANGE_BLOCKS = 16  # the fewest 32-key blocks that a range of a prompt portion's keys is worth a workgroup of its own
+PORTION_SINGLE_SET_BLOCKS = 128  # 32-key blocks of the longest row from which a workgroup is one set of waves instead of two
+DECODE_WAVES_PER_UNIT = 4  # decode rows' keys are cut into ranges until about this many waves per compute unit are at work
+LONG_ROW_KEYS = 8192  # rows that may reach this many keys get up to 32 ranges instead of 16
+
+
+@dataclass
+class LaunchPlan:
+    tiles: torch.Tensor  # int32 [n_tiles, 8]
+    hp: int
+    splits: int
+    workspace: tuple | None
+    qt: int = 1
+    coop: bool = False
+
+
+def launch_plans(ctx, group: int, kv_heads: int, head_dim: int) -> list[LaunchPlan]:
+    """How the matrix-core attention kernel is launched for a mixer with ``group`` query heads per key/value head, over
+    the tile lists of the batch: prompt portions as 32-token tiles of one head, their keys cut into ranges when there
+    are too few tiles to fill the GPU and many keys (a short portion late in a long prompt); decode rows with all heads
+    of a group in one tile and the keys cut into ranges so that the launch fills the GPU."""
+    plans = []  # made afresh per call: the workspace lives in the caller's arena scope
+    units = ops.compute_units(ctx.token_ids.device)
+    if ctx.n_chunk_tiles:
+        tokens = ctx.chunk_tiles_tokens
+        wgs = ctx.n_chunk_tiles * kv_heads * -(-group // 4)
+        blocks = -(-ctx.max_chunk_kv // 32)
+        # fewer workgroups than compute units (one fits a unit): cut the keys into ranges
+        splits = max(1, min(16, units // wgs, blocks // PORTION_RANGE_BLOCKS))
+        ws = None
+        if splits > 1:
+            cols = ctx.n_chunk_tiles * tokens * kv_heads * group
+            ws = (ctx.arena.take((cols * splits * head_dim,), torch.float32), ctx.arena.take((cols * splits * 2,), torch.float32))
+        # many workgroups with long rows of keys: one set of four waves per workgroup, two workgroups to a compute unit,
+        # each with a barrier of its own (4 to 8% faster from 4,096 keys on; slower for short rows)
+        single = splits == 1 and wgs >= 2 * units and blocks >= PORTION_SINGLE_SET_BLOCKS
+        plans.append(LaunchPlan(ctx.chunk_tiles, 1, splits, ws, qt=tokens // 16, coop=single))
+    if ctx.n_decode_tiles:
+        hp = 1
+        while hp < min(group, 16):
+            hp *= 2
+        # decode is bound by the latency of each wave's chain of loads: the four waves of a workgroup share a tile, and
+        # the keys are cut into ranges until about a thousand waves are at work
+        # (up to 32 ranges where requests may reach 8,192 keys and the tiles are few, a single request say: at 131,072
+        # keys 86 against 132 us a layer; the kernel leaves the ranges beyond the sixteenth empty for shorter rows,
+        # and where no request can be that long they are not launched: they would cost a captured step 1%)
+        items = ctx.n_decode_tiles * kv_heads * -(-group // hp)
+        splits = max(1, min(32 if ctx.max_kv_len >= LONG_ROW_KEYS else 16, DECODE_WAVES_PER_UNIT * units // (4 * items)))
+        if not ctx.captured:
+            splits = max(1, min(splits, -(-ctx.max_kv_len // 256)))
+        ws = None
+        if splits > 1:
+            cols = ctx.n_decode_tiles * (16 // hp) * kv_heads * group
+            ws = (ctx.arena.take((cols * splits * head_dim,), torch.float32), ctx.arena.take((cols * splits * 2,), torch.float32))
+        plans.append(LaunchPlan(ctx.decode_tiles, hp, splits, ws, coop=True))
+    return plans
 
 
 class Attention:
     graph_safe = True
     ends_in_residual = True  # forward takes residual=IntoResidual
+    takes_layouts = True  # load takes which copies of its matrices to keep
 
     def __init__(self, spec, prefix: str) -> None:
         if spec.heads % spec.kv_heads:
@@ -48,8 +109,9 @@ class Attention:
             **self.position.wanted(),
         }
 
-    def load(self, get, dtype, device) -> None:
+    def load(self, get, dtype, device, layouts: str = "both") -> None:
         s = self.spec
+        plain = layouts == "both"
         q, k, v, o = self._names
         rows = (s.heads + 2 * s.kv_heads) * s.head_dim
         wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
@@ -66,11 +128,14 @@ class Attention:
         if dtype == torch.bfloat16 and s.hidden % 8 == 0 and s.head_dim % 16 == 0 and rot % 16 == 0:
             self.wqkv_rope = ops.TiledWeight(wqkv, ops.qkv_rope_row_order(s.heads, s.kv_heads, s.head_dim, rot))
         # (without the plain layout the stacked matrix is also kept tiled in its own row order, for more than 16 rows)
-        self.wqkv = LinearWeight(wqkv, tiled=self.wqkv_rope is None or not Layouts.keep_plain)
-        self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous())
+        self.wqkv = LinearWeight(wqkv, keep_plain=plain, tiled=self.wqkv_rope is None or not plain)
+        self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous(), keep_plain=plain)
 
     def cache_need(self):
         return PagedNeed(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
+
+    def max_positions(self) -> int | None:
+        return self.position.max_positions
 
     def links_norms(self, rows: int) -> bool:
         """Whether, for this many rows, ``forward`` takes a ``PreNormed`` input and an ``IntoResidual`` ending."""
@@ -96,7 +161,7 @@ class Attention:
         page = cache.k.shape[2]
         if ops.mfma_attention_takes(x.dtype, s.head_dim, page):
             group = s.heads // s.kv_heads
-            for plan in ctx.attention_plans(group, s.kv_heads, s.head_dim):
+            for plan in launch_plans(ctx, group, s.kv_heads, s.head_dim):
                 ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim,
                                    s.softmax_scale, window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace,
                                    qt=plan.qt, coop=plan.coop)

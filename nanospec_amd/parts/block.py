@@ -12,18 +12,15 @@ from ..kernels import ops
 from . import registry
 from .linear import IntoResidual
 
-_MIXER_PREFIX = {"attention": "self_attn."}
-_FFN_PREFIX = {"swiglu": "mlp."}
-
-
 class PreNormBlock:
     def __init__(self, spec, prefix: str | None = None) -> None:
         p = spec.prefix if prefix is None else prefix
         self.spec = spec
-        self.mixer_norm = registry.build("norm", spec.mixer_norm, p + "input_layernorm.weight")
-        self.mixer = registry.build("mixer", spec.mixer, p + _MIXER_PREFIX.get(spec.mixer.kind, spec.mixer.kind + "."))
-        self.ffn_norm = registry.build("norm", spec.ffn_norm, p + "post_attention_layernorm.weight")
-        self.ffn = registry.build("ffn", spec.ffn, p + _FFN_PREFIX.get(spec.ffn.kind, spec.ffn.kind + "."))
+        under = lambda given, part: p + (given if given is not None else part.kind + ".")
+        self.mixer_norm = registry.build("norm", spec.mixer_norm, p + spec.mixer_norm_name)
+        self.mixer = registry.build("mixer", spec.mixer, under(spec.mixer_prefix, spec.mixer))
+        self.ffn_norm = registry.build("norm", spec.ffn_norm, p + spec.ffn_norm_name)
+        self.ffn = registry.build("ffn", spec.ffn, under(spec.ffn_prefix, spec.ffn))
         self.parts = (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
 
     @property
@@ -36,12 +33,28 @@ class PreNormBlock:
             out.update(p.wanted())
         return out
 
-    def load(self, get, dtype, device) -> None:
+    def load(self, get, dtype, device, layouts: str = "both") -> None:
         for p in self.parts:
-            p.load(get, dtype, device)
+            if getattr(p, "takes_layouts", False):
+                p.load(get, dtype, device, layouts)
+            else:
+                p.load(get, dtype, device)
+
+    takes_layouts = True
 
     def cache_need(self):
         return self.mixer.cache_need()
+
+    def max_positions(self) -> int | None:
+        """The positions the block's parts can encode; None if nothing bounds them."""
+        limits = [p.max_positions() for p in self.parts if hasattr(p, "max_positions")]
+        limits = [n for n in limits if n is not None]
+        return min(limits) if limits else None
+
+    @property
+    def entry_norm(self):
+        """The norm that reads what the block before this one left (for blocks that ``links_blocks``)."""
+        return self.mixer_norm
 
     links_blocks = True  # forward takes next_norm, next_sums and next_carry
 

@@ -19,13 +19,11 @@ import torch
 
 from ..kernels import ops
 
-class Layouts:
-    """Which copies of a bfloat16 weight matrix are kept: the re-laid one that the streaming kernels read is always
-    there; the plain one, which the library's products for many rows read, only if ``keep_plain``.  Without it many rows
-    run in slices of 64 through the hand-written kernels: slower prompts, half the memory.  Set by ``DecoderModel.load``
-    before the parts load."""
-
-    keep_plain = True
+# Which copies of a bfloat16 weight matrix a model keeps (``DecoderModel.load(..., layouts=)``; parts that say
+# ``takes_layouts`` are told at load time): the re-laid one that the streaming kernels read is always there; the plain one,
+# which the library's products for many rows read, only with "both".  With "tiled" many rows run in blocks through the
+# hand-written kernels: slower prompts, half the memory.
+LAYOUTS = ("both", "tiled")
 
 
 STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured
@@ -55,11 +53,10 @@ class IntoResidual:
 
 
 class LinearWeight:
-    def __init__(self, w: torch.Tensor, keep_plain: bool | None = None, tiled: bool = True) -> None:
+    def __init__(self, w: torch.Tensor, keep_plain: bool = True, tiled: bool = True) -> None:
         """``w``: [out, in] on the GPU in the compute dtype.  ``tiled=False``: the caller streams this matrix with a
-        kernel and a layout of its own for few rows, so only the plain layout is kept here.  ``keep_plain``: see
-        ``Layouts`` (None: its setting)."""
-        keep_plain = Layouts.keep_plain if keep_plain is None else keep_plain
+        kernel and a layout of its own for few rows, so only the plain layout is kept here.  ``keep_plain=False``: only the
+        re-laid copy is kept (see ``LAYOUTS``)."""
         self.n, self.k = w.shape
         self.dtype = w.dtype
         fast = w.dtype == torch.bfloat16 and self.k % 8 == 0
@@ -149,8 +146,7 @@ class LinearWeight:
 class GatedWeights:
     """Gate and up matrices of a gated feed-forward: silu(x @ Wg^T) * (x @ Wu^T) in one pass over x."""
 
-    def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_plain: bool | None = None) -> None:
-        keep_plain = Layouts.keep_plain if keep_plain is None else keep_plain
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_plain: bool = True) -> None:
         self.inter, self.k = gate.shape
         self.dtype = gate.dtype
         fast = gate.dtype == torch.bfloat16 and self.k % 8 == 0

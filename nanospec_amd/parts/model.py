@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights import source as wsource
 from . import registry
-from .linear import Layouts, LinearWeight
+from .linear import LAYOUTS, LinearWeight
 from .needs import PagedNeed, StateNeed
 
 
@@ -37,6 +37,7 @@ class DecoderModel:
         self.embed: torch.Tensor | None = None
         self.head: LinearWeight | None = None
         self.dtype = self.device = None
+        self._max_positions = "?"  # not asked yet
         # what every entry of the run order keeps in the cache
         self.cache_needs = [self.layers[c.layer].cache_need() if c.cache_from is None else None for c in spec.run_order]
 
@@ -51,13 +52,13 @@ class DecoderModel:
         """Check the source against what the model wants (one error that lists everything wrong), then read
         each tensor once.  A head that is absent is the embedding table if the configuration ties them
         (reference: model/loader.py:62-70).  ``layouts``: "both" keeps every bfloat16 matrix in two layouts
-        (``parts.linear.Layouts``), "tiled" only in the re-laid one, "auto" chooses by the memory that is free."""
+        (``parts.linear.LAYOUTS``), "tiled" only in the re-laid one, "auto" chooses by the memory that is free."""
         spec = self.spec
         full = self.wanted()
         wanted = {k: v[0] for k, v in full.items()}
         wsource.check(source, wanted, optional={spec.head_name} if spec.tie_head else frozenset())
         self.dtype, self.device = dtype, torch.device(device)
-        if layouts not in ("auto", "both", "tiled"):
+        if layouts != "auto" and layouts not in LAYOUTS:
             raise ValueError(f"layouts={layouts!r}: use 'auto', 'both' or 'tiled'")
         if layouts == "auto":
             size = torch.finfo(dtype).bits // 8
@@ -67,7 +68,7 @@ class DecoderModel:
             if layouts == "tiled" and dtype == torch.bfloat16:
                 print(f"[nanospec_amd] {linear / 2**30:.0f} GiB of matrices, {free / 2**30:.0f} GiB free: keeping one layout; "
                       "steps of many tokens will be slower", file=sys.stderr, flush=True)
-        Layouts.keep_plain = layouts == "both"
+        self.layouts = layouts
         get = source.get
         self.embed = get(spec.embed_name).to(device=device, dtype=dtype).contiguous()
         if spec.head_name in source.names():
@@ -75,9 +76,31 @@ class DecoderModel:
         else:
             self.head = LinearWeight(self.embed, keep_plain=False)  # the embedding table is the head
         for layer in self.layers:
-            layer.load(get, dtype, device)
+            if getattr(layer, "takes_layouts", False):
+                layer.load(get, dtype, device, layouts)
+            else:
+                layer.load(get, dtype, device)
         self.final_norm.load(get, dtype, device)
+        # whoever runs the model works on a stream of their own: everything that loading enqueued (copies, re-laying of
+        # matrices, random draws) is finished before anyone can read it
+        torch.cuda.synchronize(self.device)
         return self
+
+    # ------------------------------------------------------------------ positions
+
+    @property
+    def max_positions(self) -> int | None:
+        """The positions the model's parts can encode; None if nothing bounds them."""
+        if self._max_positions == "?":
+            limits = [layer.max_positions() for layer in self.layers if hasattr(layer, "max_positions")]
+            limits = [n for n in limits if n is not None]
+            self._max_positions = min(limits) if limits else None
+        return self._max_positions
+
+    def check_positions(self, last_position: int) -> None:
+        limit = self.max_positions
+        if limit is not None and last_position >= limit:
+            raise ValueError(f"position {last_position} is beyond the model's {limit} positions")
 
     # ------------------------------------------------------------------ one pass over the given tokens
 
@@ -98,7 +121,7 @@ class DecoderModel:
             layer = self.layers[call.layer]
             if getattr(layer, "links_blocks", False) and i + 1 < len(order):
                 # the norm that reads this block's result is the next block's first
-                nxt = getattr(self.layers[order[i + 1].layer], "mixer_norm", None)
+                nxt = getattr(self.layers[order[i + 1].layer], "entry_norm", None)
                 out = layer.forward(ctx, resid, pending, caches[i], call.cache_from is None, delta, next_norm=nxt, next_sums=sums,
                                     next_carry=carry)
             else:

@@ -14,20 +14,28 @@ What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are 
                                                   stream into buffers taken from ctx.arena
   norm         forward(ctx, resid=None, x=None, rows=None, write_resid=False, out=None)
                                                   normalise resid + x (the sum optionally stored back)
-  position     an object the mixer that owns it knows how to use (rope: ``inv_freq`` on the device)
+  position     an object the mixer that owns it knows how to use (rope: ``inv_freq`` on the device, ``rotary_dim``,
+               ``max_positions``: an int or None)
   mixer        cache_need() -> PagedNeed | StateNeed | None
                forward(ctx, x, cache, owns_cache, out=None) -> [tokens, hidden]
   ffn          forward(ctx, x, out=None) -> [tokens, hidden]
-  block        forward(ctx, resid, delta, cache, owns_cache, delta_out) -> None
+  block        __init__(spec, None): the spec carries the layer's tensor-name prefix and its parts' names
+               cache_need(); forward(ctx, resid, delta, cache, owns_cache, delta_out) -> None
                                                   resid is updated in place; the not yet added output of
                                                   the block's last part is left in delta_out
+
+Optional:
+  mixer, block max_positions() -> int | None      the positions it can encode (the engine refuses requests beyond the
+                                                  smallest limit of a model's layers)
+  any part     takes_layouts = True: load(get, dtype, device, layouts) with layouts "both" | "tiled"
+                                                  (which copies of a bfloat16 matrix to keep, ``parts.linear.LAYOUTS``)
 
 Optional, for parts whose products can do the work of the RMS norms around them (``parts.linear.IntoResidual``):
   norm         links_products = True, weight, spec.eps
   mixer, ffn   ends_in_residual = True: forward(..., residual=IntoResidual) -> PreNormed | PartialSums | Added | tensor;
                links_norms(rows) -> bool: x may be a PreNormed
-  block        links_blocks = True; forward(..., next_norm=None, next_sums=None, next_carry=None) -> None or one of
-               those three
+  block        links_blocks = True; entry_norm (the norm that reads the block's input);
+               forward(..., next_norm=None, next_sums=None, next_carry=None) -> None or one of those three
 """
 
 from __future__ import annotations

@@ -12,6 +12,7 @@ from .linear import GatedWeights, LinearWeight
 class SwiGLU:
     graph_safe = True
     ends_in_residual = True  # forward takes residual=IntoResidual
+    takes_layouts = True  # load takes which copies of its matrices to keep
 
     def __init__(self, spec, prefix: str) -> None:
         self.spec, self.prefix = spec, prefix
@@ -26,11 +27,12 @@ class SwiGLU:
             p + "down_proj.weight": ((s.hidden, s.intermediate), "linear"),
         }
 
-    def load(self, get, dtype, device) -> None:
+    def load(self, get, dtype, device, layouts: str = "both") -> None:
         s, p = self.spec, self.prefix
+        plain = layouts == "both"
         self.gate_up = GatedWeights(get(p + "gate_proj.weight").to(device=device, dtype=dtype),
-                                    get(p + "up_proj.weight").to(device=device, dtype=dtype))
-        self.down = LinearWeight(get(p + "down_proj.weight").to(device=device, dtype=dtype).contiguous())
+                                    get(p + "up_proj.weight").to(device=device, dtype=dtype), keep_plain=plain)
+        self.down = LinearWeight(get(p + "down_proj.weight").to(device=device, dtype=dtype).contiguous(), keep_plain=plain)
 
     def links_norms(self, rows: int) -> bool:
         """Whether, for this many rows, ``forward`` takes a ``PreNormed`` input and an ``IntoResidual`` ending."""

@@ -18,6 +18,18 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
+LLAMA_NAMES = dict(mixer_norm_name="input_layernorm.weight", ffn_norm_name="post_attention_layernorm.weight")
+
+
+def llama_block(prefix, norm1, mixer, norm2, ffn):
+    """A pre-norm block whose norms, attention and SwiGLU carry the Llama checkpoints' names; toy parts get their kind."""
+    from nanospec_amd.config.spec import PreNormBlockSpec
+
+    return PreNormBlockSpec(prefix, norm1, mixer, norm2, ffn, **LLAMA_NAMES,
+                            mixer_prefix="self_attn." if mixer.kind == "attention" else None,
+                            ffn_prefix="mlp." if ffn.kind == "swiglu" else None)
+
+
 def make_ctx(lens, starts, tables, page, dtype, want=()):
     """A StepContext for hand-made requests: tables[b] lists the pages of request b."""
     import numpy as np
@@ -197,8 +209,8 @@ def toy_model(dtype):
     norm = RMSNormSpec(hidden, 1e-5)
     ffn = SwiGLUSpec(hidden, 80)
     attn = AttentionSpec(hidden, 3, 1, 16, RopeSpec(16, 1e4), 1 / math.sqrt(16))
-    layers = (PreNormBlockSpec("model.layers.0.", norm, PrefixMeanSpec(hidden), norm, ffn),
-              PreNormBlockSpec("model.layers.1.", norm, attn, norm, ffn))
+    layers = (llama_block("model.layers.0.", norm, PrefixMeanSpec(hidden), norm, ffn),
+              llama_block("model.layers.1.", norm, attn, norm, ffn))
     spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers,
                      (LayerCall(0), LayerCall(1), LayerCall(1), LayerCall(1, cache_from=1)), norm, "model.norm.weight", "lm_head.weight", True)
     net = DecoderModel(spec)
@@ -350,8 +362,8 @@ def test_toy_routed_feed_forward_and_toy_position_in_one_layer_only():
     register("position", "harmonic", HarmonicRotation)
     hidden, vocab, hd = 40, 61, 32
     norm = RMSNormSpec(hidden, 1e-5)
-    layers = (PreNormBlockSpec("model.layers.0.", norm, AttentionSpec(hidden, 2, 2, hd, RopeSpec(hd, 1e4), 1 / math.sqrt(hd)), norm, SwiGLUSpec(hidden, 56)),
-              PreNormBlockSpec("model.layers.1.", norm, AttentionSpec(hidden, 2, 1, hd, HarmonicRotationSpec(16), 0.25), norm, TopOneExpertsSpec(hidden, 24, 3)))
+    layers = (llama_block("model.layers.0.", norm, AttentionSpec(hidden, 2, 2, hd, RopeSpec(hd, 1e4), 1 / math.sqrt(hd)), norm, SwiGLUSpec(hidden, 56)),
+              llama_block("model.layers.1.", norm, AttentionSpec(hidden, 2, 1, hd, HarmonicRotationSpec(16), 0.25), norm, TopOneExpertsSpec(hidden, 24, 3)))
     spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers, (LayerCall(0), LayerCall(1)), norm, "model.norm.weight", "lm_head.weight", False)
     net = DecoderModel(spec)
     wanted = net.wanted()
@@ -396,3 +408,113 @@ def test_toy_routed_feed_forward_and_toy_position_in_one_layer_only():
         want = torch.cat([refs[r][s:e] for r, s, e in entries])
         err = ((out.cpu() - want).abs().amax(-1) / want.abs().amax(-1)).max()
         assert err < 1e-4, (entries, float(err))
+
+
+# ------------------------------------------------------- a toy block of another shape, and tensor names of another origin
+
+
+@dataclass(frozen=True)
+class ParallelBlockSpec:
+    """x = x + mixer(norm(x)) + feed_forward(norm(x)): one norm whose output both parts read."""
+
+    kind: ClassVar[str] = "parallel"
+    prefix: str
+    norm: object
+    mixer: object
+    ffn: object
+
+
+class ParallelBlock:
+    graph_safe = False  # the sum of the two parts is a torch operation
+
+    def __init__(self, spec, prefix=None):
+        from nanospec_amd.parts import build
+
+        p = spec.prefix
+        self.norm = build("norm", spec.norm, p + "ln.w")
+        self.mixer = build("mixer", spec.mixer, p + "att.")
+        self.ffn = build("ffn", spec.ffn, p + "ff.")
+        self.parts = (self.norm, self.mixer, self.ffn)
+
+    def wanted(self):
+        out = {}
+        for part in self.parts:
+            out.update(part.wanted())
+        return out
+
+    def load(self, get, dtype, device):
+        for part in self.parts:
+            part.load(get, dtype, device)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, ctx, resid, delta, cache, owns_cache, delta_out):
+        h = self.norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None)
+        a = self.mixer.forward(ctx, h, cache, owns_cache)
+        f = self.ffn.forward(ctx, h)
+        delta_out.copy_((a.float() + f.float()).to(delta_out.dtype))
+        return None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_toy_block_and_other_tensor_names(dtype):
+    """A block of another shape registered from here (one norm, mixer and feed-forward side by side, tensor names of its
+    own) before a pre-norm block whose four names are not Llama's: nothing in the framework knows either set of names."""
+    import math
+
+    from nanospec_amd.config.spec import AttentionSpec, LayerCall, ModelSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.parts import DecoderModel, register
+    from nanospec_amd.weights import DictSource, random_tensors
+
+    register("block", "parallel", ParallelBlock)
+    hidden, vocab, hd = 64, 131, 16
+    norm = RMSNormSpec(hidden, 1e-5)
+    attn = AttentionSpec(hidden, 4, 2, hd, RopeSpec(hd, 1e4, max_positions=96), 1 / math.sqrt(hd))
+    ffn = SwiGLUSpec(hidden, 96)
+    layers = (ParallelBlockSpec("h.0.", norm, attn, ffn),
+              PreNormBlockSpec("h.1.", norm, attn, norm, ffn, mixer_norm_name="ln_a.weight", mixer_prefix="mix.",
+                               ffn_norm_name="ln_b.weight", ffn_prefix="feed."))
+    spec = ModelSpec(vocab, hidden, "wte", layers, (LayerCall(0), LayerCall(1)), norm, "ln_f", "out_head", False)
+    net = DecoderModel(spec)
+    names = set(net.wanted())
+    assert {"h.0.ln.w", "h.0.att.q_proj.weight", "h.0.ff.down_proj.weight", "h.1.ln_a.weight", "h.1.mix.o_proj.weight",
+            "h.1.ln_b.weight", "h.1.feed.gate_proj.weight", "wte", "ln_f", "out_head"} <= names
+    assert not any("layernorm" in n or "self_attn" in n or "mlp" in n for n in names)
+    w = {k: (v * (5.0 if "proj" in k else 1.0)).to(dtype) for k, v in random_tensors(net.wanted(), seed=21).items()}
+    model = net.load(DictSource(w), dtype, DEV)
+    assert model.max_positions == 96
+
+    def plain(tokens):
+        t = len(tokens)
+        x = w["wte"][torch.tensor(tokens)]
+        cos, sin = pl.rotation_tables(torch.arange(t), pl.inverse_frequencies(hd, 1e4, None))
+
+        def attention(h, p):
+            q = pl.rotate(pl.linear(h, w[p + "q_proj.weight"]).view(t, 4, hd), cos, sin)
+            k = pl.rotate(pl.linear(h, w[p + "k_proj.weight"]).view(t, 2, hd), cos, sin)
+            v = pl.linear(h, w[p + "v_proj.weight"]).view(t, 2, hd)
+            return pl.linear(pl.causal_attention(q, k, v).reshape(t, -1), w[p + "o_proj.weight"])
+
+        feed = lambda h, p: pl.swiglu(h, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+        h = pl.rms_norm(x, w["h.0.ln.w"], 1e-5)
+        x = pl.residual_add(x, (attention(h, "h.0.att.").float() + feed(h, "h.0.ff.").float()).to(dtype))
+        x = pl.residual_add(x, attention(pl.rms_norm(x, w["h.1.ln_a.weight"], 1e-5), "h.1.mix."))
+        x = pl.residual_add(x, feed(pl.rms_norm(x, w["h.1.ln_b.weight"], 1e-5), "h.1.feed."))
+        return pl.rms_norm(x, w["ln_f"], 1e-5).float() @ w["out_head"].float().T
+
+    g = torch.Generator().manual_seed(8)
+    seqs = {r: torch.randint(0, vocab, (n,), generator=g).tolist() for r, n in (("a", 45), ("b", 23))}
+    refs = {r: plain(t) for r, t in seqs.items()}
+    rep = Replayer(model, 256, page_size=4)
+    for entries in ([("a", 0, 20), ("b", 0, 3)], [("a", 20, 21), ("b", 3, 23)], [("a", 21, 45)]):
+        out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(range(e - s))} for r, s, e in entries], [])
+        want = torch.cat([refs[r][s:e] for r, s, e in entries])
+        if dtype == torch.float32:
+            err = ((out.cpu() - want).abs().amax(-1) / want.abs().amax(-1)).max()
+            assert err < 1e-4, (entries, float(err))
+        else:
+            assert ulps_of_row_max(out.cpu(), want).max() <= 8, entries
+    with pytest.raises(ValueError):  # the block's mixer bounds the positions, and the model asks the block
+        rep.step([{"id": "c", "tokens": list(range(97)), "want": []}], [])

@@ -121,11 +121,107 @@ def test_whole_model_properties(tiny_folders):
     assert full.shape == (6, 256)
     # causality: a prefix's logits do not depend on what follows
     torch.testing.assert_close(pl.logits_of_sequence(w, cfg, toks[:4]), full[:4], rtol=1e-5, atol=1e-6)
-    # the last norm is applied: logits equal normed hidden times the embedding table
     cfgB, wB = pl.read_config(tiny_folders["B"]), pl.read_weights(tiny_folders["B"], torch.float32)
     assert not cfgB["tied"] and cfgB["scaling"]["factor"] == 8.0 and cfgB["kv_heads"] == 1 and cfgB["eps"] == 1e-6
     new, rows = pl.greedy_continuation(wB, cfgB, [5, 6, 7], 3)
     assert len(new) == 3 and new[0] == int(pl.logits_of_sequence(wB, cfgB, [5, 6, 7])[-1].argmax())
+
+
+# ------------------------------------------------------------------ how the parts are put together
+# No text but the reference's fixes the order of norms, sums and rotations, so each property below is one that only the
+# right arrangement has: a plausible other arrangement (a norm after the sum, a branch that reads the raw stream, a value
+# that is rotated, a last norm left out) fails at least one of them.
+
+
+def _layer_setup(name, tiny_folders, t=9):
+    cfg, w = pl.read_config(tiny_folders[name]), pl.read_weights(tiny_folders[name], torch.float32)
+    torch.manual_seed(5)
+    x = torch.randn(t, cfg["hidden"])
+    inv = pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"])
+    return cfg, dict(w), x, inv
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_layer_is_pre_norm_with_two_plain_sums(tiny_folders, name):
+    cfg, w, x, inv = _layer_setup(name, tiny_folders)
+    p = "model.layers.0."
+    cos, sin = pl.rotation_tables(torch.arange(x.shape[0]), inv)
+    out = pl.decoder_layer(x, w, p, cfg, cos, sin)
+    # (1) the norms sit in front of the parts, inside the branches: with both norm weights zero each part sees zeros and
+    #     returns zeros (no biases), and the layer is the identity.  A norm behind a sum would give zeros.
+    w0 = dict(w)
+    w0[p + "input_layernorm.weight"] = torch.zeros_like(w[p + "input_layernorm.weight"])
+    w0[p + "post_attention_layernorm.weight"] = torch.zeros_like(w[p + "post_attention_layernorm.weight"])
+    assert torch.equal(pl.decoder_layer(x, w0, p, cfg, cos, sin), x)
+    # (2) each branch is added once, unscaled: without the feed-forward (down = 0) the layer's change of the stream is
+    #     linear in the output projection, and it vanishes with it
+    wd = dict(w)
+    wd[p + "mlp.down_proj.weight"] = torch.zeros_like(w[p + "mlp.down_proj.weight"])
+    inc = pl.decoder_layer(x, wd, p, cfg, cos, sin) - x
+    wd2 = dict(wd)
+    wd2[p + "self_attn.o_proj.weight"] = 2 * w[p + "self_attn.o_proj.weight"]
+    torch.testing.assert_close(pl.decoder_layer(x, wd2, p, cfg, cos, sin) - x, 2 * inc, rtol=1e-5, atol=1e-6)
+    wd2[p + "self_attn.o_proj.weight"] = torch.zeros_like(w[p + "self_attn.o_proj.weight"])
+    assert torch.equal(pl.decoder_layer(x, wd2, p, cfg, cos, sin), x)
+    # (3) the branches read the NORMED stream: scaling the stream leaves the attention branch's output as it was (eps is
+    #     tiny beside these values), so the change of the stream stays the same while the stream is seven times larger
+    torch.testing.assert_close(pl.decoder_layer(7 * x, wd, p, cfg, cos, sin) - 7 * x, inc, rtol=1e-3, atol=1e-5)
+    # (4) the feed-forward reads the stream AFTER the attention's sum: it equals the feed-forward alone applied to it
+    mid = x + inc
+    wa = dict(w)
+    wa[p + "self_attn.o_proj.weight"] = torch.zeros_like(w[p + "self_attn.o_proj.weight"])
+    torch.testing.assert_close(out, pl.decoder_layer(mid, wa, p, cfg, cos, sin), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_layer_rotates_queries_and_keys_but_not_values(tiny_folders, name):
+    """Only distances count: with every position shifted by the same amount the layer's output is the same.  That holds
+    if queries and keys are turned alike and values are not; a rotated value, or a rotation of one of q and k only,
+    changes the output with the shift."""
+    cfg, w, x, inv = _layer_setup(name, tiny_folders)
+    p = "model.layers.0."
+    t = x.shape[0]
+    base = pl.decoder_layer(x, w, p, cfg, *pl.rotation_tables(torch.arange(t), inv))
+    far = pl.decoder_layer(x, w, p, cfg, *pl.rotation_tables(torch.arange(t) + 41, inv))
+    torch.testing.assert_close(far, base, rtol=1e-4, atol=1e-5)
+    # and the rotation is there at all: reversing the order of the positions changes the output
+    back = pl.decoder_layer(x, w, p, cfg, *pl.rotation_tables(torch.arange(t - 1, -1, -1), inv))
+    assert not torch.allclose(back, base, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_model_without_branches_is_last_norm_and_head(tiny_folders, name):
+    """With every output and down projection zero the layers pass the embedding through, and the logits must be the
+    library's RMS norm of the embedding rows times the head: the last norm is applied, once, with the model's eps, and
+    the head is the tied table or the head of its own."""
+    cfg, w = pl.read_config(tiny_folders[name]), dict(pl.read_weights(tiny_folders[name], torch.float32))
+    for k in list(w):
+        if k.endswith("o_proj.weight") or k.endswith("down_proj.weight"):
+            w[k] = torch.zeros_like(w[k])
+    toks = [3, 99, 17, 17, 42]
+    emb = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    normed = F.rms_norm(emb, (cfg["hidden"],), w["model.norm.weight"], cfg["eps"])
+    head = w["model.embed_tokens.weight"] if cfg["tied"] else w["lm_head.weight"]
+    got = pl.logits_of_sequence(w, cfg, toks)
+    torch.testing.assert_close(got, normed @ head.T, rtol=1e-5, atol=1e-6)
+    w2 = dict(w)
+    w2["model.norm.weight"] = 2 * w["model.norm.weight"]
+    torch.testing.assert_close(pl.logits_of_sequence(w2, cfg, toks), 2 * got, rtol=1e-5, atol=1e-6)
+    assert torch.equal(got[2], got[3])  # equal tokens, nothing mixes positions: equal rows
+
+
+def test_layers_run_in_order_and_each_once(tiny_folders):
+    """Swapping two layers' weights changes the logits; and the model is the layers applied in turn to the embedding."""
+    cfg, w = pl.read_config(tiny_folders["B"]), pl.read_weights(tiny_folders["B"], torch.float32)
+    toks = [5, 600, 7, 123, 9, 9, 31]
+    full = pl.logits_of_sequence(w, cfg, toks)
+    x = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    cos, sin = pl.rotation_tables(torch.arange(len(toks)), pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"]))
+    for i in range(cfg["layers"]):
+        x = pl.decoder_layer(x, w, f"model.layers.{i}.", cfg, cos, sin)
+    torch.testing.assert_close(full, pl.rms_norm(x, w["model.norm.weight"], cfg["eps"]) @ w["lm_head.weight"].T)
+    swapped = {k.replace("layers.0.", "layers.X.").replace("layers.1.", "layers.0.").replace("layers.X.", "layers.1."): v for k, v in w.items()}
+    assert not torch.allclose(pl.logits_of_sequence(swapped, cfg, toks), full, rtol=1e-3, atol=1e-4)
 
 
 def test_processed_logprobs_vectors():

@@ -61,13 +61,44 @@ def check(ours: torch.Tensor, ref: torch.Tensor, dtype, what: str):
         assert u.max() <= 8, f"{what}: {u.max():.2f} bf16 ulps of the row's largest logit (median {u.median():.2f})"
 
 
-def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, link_norms=True):
+def churn(manager, rounds=200, seed=0):
+    """Random reservations and releases before a run (reference: tests/test_correctness.py:25-50), so that the free list
+    is in no order and every request's pages lie scattered over the pool."""
+    import random
+
+    rng = random.Random(seed)
+    held = []
+    for i in range(rounds):
+        if held and (rng.random() < 0.5 or manager.slots.num_free == 0 or manager.num_free(0) < 8):
+            manager.release(held.pop(rng.randrange(len(held))))
+        else:
+            rid = f"churn{i}"
+            manager.admit(rid)
+            n = rng.randint(1, 7 * manager.page_size)
+            manager.reserve(rid, n)
+            manager.commit(rid, n)
+            held.append(rid)
+    rng.shuffle(held)
+    for rid in held:
+        manager.release(rid)
+    manager.check()
+
+
+def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, link_norms=True, churned=False):
     from nanospec_amd.engine.replay import Replayer
 
     rep = Replayer(model, max_tokens, page_size=page, use_graphs=graphs)
     rep.runner.link_norms = link_norms
+    if churned:
+        churn(rep.manager)
+        rep.scattered = 0
     for step, w in zip(steps, where):
         out = rep.step(step["entries"], step["end"])
+        if churned:
+            for e in step["entries"]:
+                if e["id"] in rep.manager:
+                    table = rep.manager.get(e["id"]).tables[0]
+                    rep.scattered += sum(1 for a, b in zip(table, table[1:]) if a is not None and b is not None and abs(b - a) != 1)
         if not w:
             assert out is None
             continue
@@ -106,6 +137,18 @@ def test_schedules_match_plain(tiny_folders, name, dtype, schedule):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_schedule_on_a_churned_pool(tiny_folders, name, dtype):
+    """reference tests/test_correctness.py:25-50: two hundred random reservations and releases come first, so the pages a
+    request gets are neither consecutive nor in rising order; the mixed schedule on so few pages that they are used again."""
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    steps, where, peak = traces.mixed(seqs, seed=23)
+    rep = replay(engine_model(folder, name, dtype), steps, where, plain_logits(folder, name, dtype), dtype, peak, page, churned=True)
+    assert rep.scattered > 20, "the block tables were meant to be scattered"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B"])
 def test_long_decoding_from_the_first_token(tiny_folders, name, dtype):
     """Two requests decoded one token at a time from position 0 to the model's last position: the first tokens of a
     sequence (one key, then two, ...), every page edge on the way, and errors that would build up over many steps."""
@@ -133,6 +176,64 @@ def test_graph_and_eager_decode_agree(tiny_folders, name):
     a = replay(model, steps, where, ref, torch.bfloat16, 256, page, graphs=True)
     assert a.runner._graphs, "decode steps did not replay a graph"
     replay(model, steps, where, ref, torch.bfloat16, 256, page, graphs=False)
+
+
+# requests that decode together -> the captured step they must replay: every bucket of the runner
+BUCKET_CASES = [(1, 1), (2, 2), (3, 4), (7, 8), (12, 16), (20, 32), (40, 48), (60, 64), (70, 96), (100, 128), (150, 176), (200, 208),
+                (230, 240), (250, 256)]
+
+
+def test_bucket_cases_cover_every_bucket():
+    from nanospec_amd.engine.runner import GRAPH_BUCKETS
+
+    assert [b for _, b in BUCKET_CASES] == list(GRAPH_BUCKETS)
+
+
+@pytest.mark.parametrize("n_requests,bucket", BUCKET_CASES)
+def test_every_graph_bucket_against_plain(tiny_folders, n_requests, bucket):
+    """reference tests/test_graphs.py:43-72, for every bucket: so many requests decode together that the step replays the
+    captured graph of that many rows (pad rows included), and every row's logits are the plain implementation's.  Above
+    128 rows the step runs other code (the library's products, the sum in the product, norms of their own)."""
+    from nanospec_amd.engine.replay import Replayer
+
+    name = "B"
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    vocab = TINY[name]["cfg"]["vocab_size"]
+    cfg, w = pl.read_config(folder), pl.read_weights(folder, torch.bfloat16)
+    model = engine_model(folder, name, torch.bfloat16)
+    decoded = 3
+    seqs = {f"q{i}": random_tokens(2 + (5 * i) % 17 + decoded, vocab, 4000 + i) for i in range(n_requests)}
+    ref = {r: pl.logits_of_sequence(w, cfg, t, torch.bfloat16) for r, t in seqs.items()}
+    rep = Replayer(model, sum(-(-len(t) // page) * page for t in seqs.values()) + page, page_size=page, max_live=n_requests)
+    ids = list(seqs)
+    for at in range(0, n_requests, 24):  # the prompts, two dozen requests to a step, nothing wanted
+        rep.step([{"id": r, "tokens": seqs[r][:-decoded], "want": []} for r in ids[at : at + 24]], [])
+    for d in range(decoded, 0, -1):
+        entries = [{"id": r, "tokens": [seqs[r][-d]], "want": [0]} for r in ids]
+        out = rep.step(entries, ids if d == 1 else [])
+        assert rep.runner.last_used_graph and bucket in rep.runner._graphs
+        want = torch.stack([ref[r][len(seqs[r]) - d] for r in ids])
+        check(out, want, torch.bfloat16, f"{n_requests} requests, {d} tokens before their end")
+    rep.manager.check()
+
+
+def test_graph_step_in_which_only_some_rows_want_logits(tiny_folders):
+    """A decode-only step replays the captured graph, which computes every row's logits; what comes back is the rows that
+    were asked for, in the order of the entries."""
+    from nanospec_amd.engine.replay import Replayer
+
+    name = "A"
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ids = list(seqs)[1:5]
+    for dtype in (torch.float32, torch.bfloat16):
+        ref = plain_logits(folder, name, dtype)
+        rep = Replayer(engine_model(folder, name, dtype), 512, page_size=page)
+        rep.step([{"id": r, "tokens": seqs[r][:9], "want": []} for r in ids], [])
+        for p, wanting in ((9, [0, 2]), (10, [1, 2, 3]), (11, [3]), (12, [0, 1, 2, 3])):
+            out = rep.step([{"id": r, "tokens": [seqs[r][p]], "want": [0] if i in wanting else []} for i, r in enumerate(ids)], [])
+            assert rep.runner.last_used_graph
+            check(out, torch.stack([ref[ids[i]][p] for i in wanting]), dtype, f"position {p}, rows {wanting}")
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
@@ -173,10 +274,10 @@ def test_norms_as_kernels_of_their_own(tiny_folders, name, schedule):
 def test_prompt_portions_with_their_keys_cut_into_ranges(tiny_folders, name, schedule, monkeypatch):
     """A short portion late in a long prompt has its keys cut into ranges that workgroups of their own walk.  The tiny
     models' prompts are too short for that by the engine's own rule, so the rule's threshold is lowered to one block."""
-    from nanospec_amd.engine import context
     from nanospec_amd.kernels import ops
+    from nanospec_amd.parts import attention
 
-    monkeypatch.setattr(context, "CHUNK_RANGE_BLOCKS", 1)
+    monkeypatch.setattr(attention, "PORTION_RANGE_BLOCKS", 1)
     folder, page = tiny_folders[name], TINY[name]["page"]
     seqs = sequences(name)
     ref = plain_logits(folder, name, torch.bfloat16)
@@ -204,19 +305,17 @@ def test_one_weight_layout_only(tiny_folders, name):
     """Without the plain layout (models that fill the memory) steps of many tokens run in slices through the streaming
     kernels: same logits."""
     from nanospec_amd.loader import load_model
-    from nanospec_amd.parts.linear import Layouts
 
     folder, page = tiny_folders[name], TINY[name]["page"]
     seqs = sequences(name)
     ref = plain_logits(folder, name, torch.bfloat16)
-    try:
-        model = load_model(folder, dtype=torch.bfloat16, layouts="tiled")
-        assert model.layers[0].ffn.down.plain is None and model.layers[0].ffn.gate_up.stacked is None
-        for make in (traces.whole, traces.tail_decoded):
-            steps, where = make(seqs)
-            replay(model, steps, where, ref, torch.bfloat16, 256, page)
-    finally:
-        Layouts.keep_plain = True
+    model = load_model(folder, dtype=torch.bfloat16, layouts="tiled")
+    assert model.layers[0].ffn.down.plain is None and model.layers[0].ffn.gate_up.stacked is None
+    both = load_model(folder, dtype=torch.bfloat16, layouts="both")  # a second model in the process keeps its own choice
+    assert both.layers[0].ffn.down.plain is not None and model.layers[0].mixer.wo.plain is None
+    for make in (traces.whole, traces.tail_decoded):
+        steps, where = make(seqs)
+        replay(model, steps, where, ref, torch.bfloat16, 256, page)
 
 
 def test_trace_run_program(tiny_folders, tmp_path):
@@ -309,3 +408,84 @@ def test_real_shape_slice_matches_plain(llama_1b_slice, dtype, request):
         assert seen["unadded"] > 0 and seen["linked"] > 0, seen
     else:
         assert seen == {"unadded": 0, "linked": 0}
+
+
+@pytest.fixture(scope="module")
+def llama_8b_slice(tmp_path_factory):
+    """Two layers of the Llama-3.1-8B shape (width 4096, 32 heads over 8 key/value heads of 128, feed-forward 14336,
+    vocabulary 128256, a head of its own, llama3 scaling with factor 8), random weights: the sizes that the benchmark runs."""
+    from nanospec_amd.config import LlamaConfig
+    from nanospec_amd.weights import write_model_folder
+
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+               num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-5, rope_theta=500000.0,
+               max_position_embeddings=131072, tie_word_embeddings=False,
+               rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    return write_model_folder(tmp_path_factory.mktemp("llama8b") / "m", LlamaConfig.from_hf(cfg), seed=4, dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_benchmark_shape_slice_matches_plain(llama_8b_slice, dtype):
+    """The layer sizes of the benchmark end to end: a portion of 280 tokens, a mixed step, decoding with 8 live requests
+    (captured step; norms folded into the products), prompts of 56 more requests, decoding with 64 live requests (the
+    17-to-64-row kernels, unadded ranges into the norms, the library's q/k/v product), and a step of 63 decode rows beside
+    a new prompt."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.loader import load_model
+
+    folder = llama_8b_slice
+    cfg = pl.read_config(folder)
+    w = pl.read_weights(folder, dtype)
+    # matrices as 32-bit tensors that hold the stored (bfloat16-rounded) values: the plain functions convert a matrix at
+    # every use, which at these sizes would take most of the test's time; vectors (norm weights) keep the dtype, which
+    # decides how the norm rounds
+    w = {k: (v if v.dim() == 1 else v.float()) for k, v in w.items()}
+    vocab = cfg["vocab"]
+    lengths = {"r0": 305, **{f"r{i}": 6 + i % 7 + 5 for i in range(1, 8)}, **{f"r{i}": 4 + i % 9 + 3 for i in range(8, 64)}, "r64": 40}
+    seqs = {r: random_tokens(n, vocab, 7000 + i) for i, (r, n) in enumerate(lengths.items())}
+    inv = pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"])
+    hidden = {}
+    for r, toks in seqs.items():  # the stream after the last layer, every position
+        x = w["model.embed_tokens.weight"][torch.tensor(toks)].to(dtype)
+        cos, sin = pl.rotation_tables(torch.arange(len(toks)), inv)
+        for i in range(cfg["layers"]):
+            x = pl.decoder_layer(x, w, f"model.layers.{i}.", cfg, cos, sin)
+        hidden[r] = x
+
+    def plain_rows(places):
+        x = torch.stack([hidden[r][p] for r, p in places])
+        return pl.rms_norm(x, w["model.norm.weight"], cfg["eps"]).float() @ w["lm_head.weight"].T
+
+    model = load_model(folder, dtype=dtype)
+    rep = Replayer(model, 305 + 64 * 64 + 64, page_size=16, max_live=65)
+    at = {r: 0 for r in seqs}
+
+    def step(parts, graph=None):
+        """parts: (request, tokens it brings, places among them whose logits are compared)"""
+        entries, places = [], []
+        for r, n, wants in parts:
+            entries.append({"id": r, "tokens": seqs[r][at[r] : at[r] + n], "want": list(wants)})
+            places += [(r, at[r] + i) for i in wants]
+            at[r] += n
+        out = rep.step(entries, [])
+        if graph is not None:
+            assert rep.runner.last_used_graph and graph in rep.runner._graphs
+        if places:
+            check(out, plain_rows(places), dtype, str([(r, n) for r, n, _ in parts][:4]))
+        else:
+            assert out is None
+
+    first8 = [f"r{i}" for i in range(8)]
+    step([("r0", 280, [0, 255, 279])])
+    step([("r0", 20, [19])] + [(r, lengths[r] - 5, [lengths[r] - 6]) for r in first8[1:]])
+    for _ in range(2):
+        step([(r, 1, [0]) for r in first8], graph=8)
+    rest = [f"r{i}" for i in range(8, 64)]
+    step([(r, lengths[r] - 3, []) for r in rest[:28]])
+    step([(r, lengths[r] - 3, [lengths[r] - 4]) for r in rest[28:]])
+    for _ in range(2):
+        step([(r, 1, [0]) for r in first8 + rest], graph=64)
+    step([(r, 1, [0]) for r in first8[1:] + rest] + [("r64", 40, [0, 39])])
+    assert all(at[r] == lengths[r] for r in lengths if r != "r0") and at["r0"] == 304
+    rep.manager.check()

@@ -103,14 +103,49 @@ def test_token_budget_cuts_prompts_into_portions():
 
 
 def test_budget_smaller_than_the_decoding_requests():
+    """Nobody starves: with room for two of three decoding requests per step they take turns (the one that has waited
+    longest goes first), so their outputs never differ by more than one token."""
     s = Scheduler(manager(64, 4), max_admit=8, max_step_tokens=2)
-    for i in range(3):
-        s.add(req(i, 1, max_tokens=5))
+    reqs = [req(i, 1, max_tokens=5) for i in range(3)]
+    for r in reqs:
+        s.add(r)
     assert ids(run_step(s)) == [(0, 1), (1, 1)]
-    assert ids(run_step(s)) == [(0, 1), (1, 1)]  # decoding requests first; request 2 waits for room in the budget
+    assert ids(run_step(s)) == [(0, 1), (2, 1)]  # request 2 has waited longest, then request 0 by admission order
+    assert ids(run_step(s)) == [(1, 1), (2, 1)]
     while s.has_work:
         assert sum(w.n for w in run_step(s)) <= 2
+        live = [len(r.out_tokens) for r in reqs if r.state == "running"]
+        assert not live or max(live) - min(live) <= 1
+    assert all(len(r.out_tokens) == 5 for r in reqs)
     assert s.cache.num_free() == 64
+
+
+def test_a_prompt_advances_although_the_decoding_requests_fill_the_budget():
+    """Eight decoding requests and a budget of eight: an eighth of it (one token here) is kept for the oldest unfinished
+    prompt, which would otherwise wait until a decoding request finishes; the decoding requests share what is left."""
+    s = Scheduler(manager(256, 4), max_admit=16, max_step_tokens=8)
+    dec = [req(i, 1, max_tokens=60) for i in range(8)]
+    for r in dec:
+        s.add(r)
+    run_step(s)  # all eight have their one prompt token in the cache and decode from here on
+    late = req(8, 30, max_tokens=2)
+    s.add(late)
+    for _ in range(29):
+        work = run_step(s)
+        assert sum(w.n for w in work) <= 8
+        assert (8, 1) in ids(work)  # the prompt's token of this step
+    assert late.computed == 29  # its last token left, it takes turns with the others like a decoding request
+    for _ in range(4):
+        run_step(s)
+    assert late.state == "done" and len(late.out_tokens) == 2
+    assert max(len(r.out_tokens) for r in dec) - min(len(r.out_tokens) for r in dec) <= 1
+    # with a wider budget the prompt takes all that the decoding requests leave
+    s2 = Scheduler(manager(256, 4), max_admit=16, max_step_tokens=20)
+    for i in range(8):
+        s2.add(req(i, 1, max_tokens=60))
+    run_step(s2)
+    s2.add(req(8, 30, max_tokens=2))
+    assert ids(run_step(s2))[-1] == (8, 12)
 
 
 def test_preemption_when_pages_run_out():
