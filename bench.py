@@ -3,11 +3,13 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Prints ONE JSON line.  ``value`` is decoded tokens per second at batch 8 through the whole engine (scheduler,
-step function, captured graphs, sampling): every request is prefilled with 2,048 random token ids, then W untimed
-and K timed decode steps run (K = 2,048 takes the context from 2,048 to 4,096).  ``points`` holds the same at
-batch 1 and 64 over a shorter window of steps centred on context 3,072, the mean of 2,048..4,096.  ``prefill`` is
-one step of 2,048 prompt tokens of one request; ``roofline`` is the bytes a decode step must read (every weight
-once, the cache of the live requests) over its time, against 8 TB/s.
+step function, captured graphs, sampling).  The benchmark decodes from context 2,048 to 4,096; a step's time grows
+linearly with the context, so K timed steps (after W untimed ones) are taken as a window centred on context 3,072,
+the mean of 2,048..4,096, and stand for the whole run; with K >= 2,048 the whole run is timed (prompts of 2,048
+random token ids, then 2,048 decode steps).  ``metric`` and ``config`` name the contexts that were timed.  ``points``
+holds the same at batch 1 and 64 (windows of at most 256 steps) and ``points_hbm_frac`` their fractions of the
+memory roofline.  ``prefill`` is one step of 2,048 prompt tokens of one request; ``roofline`` is the bytes a decode
+step must read (every weight once, the cache of the live requests) over its time, against 8 TB/s.
 """
 
 from __future__ import annotations
@@ -132,10 +134,12 @@ def serve_run(model, cfg, n_requests: int, new_tokens: int, chunk: int, block_si
     prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lens]
     per_request = -(-(1024 + new_tokens + 1) // block_size)
     best = None
-    for _ in range(reps):  # the first pass captures the decode graphs
-        eng = Engine(model, EngineConfig(num_blocks=n_requests * per_request + 2, block_size=block_size, max_admit=n_requests,
-                                         max_running=n_requests, max_step_tokens=chunk + n_requests, prefill_chunk=chunk,
-                                         max_seq_len=1024 + new_tokens + block_size))
+    # One engine for all passes, as a server is one engine for all its requests: the first pass captures the steps' graphs
+    # (the reference captures its graphs before it serves), the later ones are timed.
+    eng = Engine(model, EngineConfig(num_blocks=n_requests * per_request + 2, block_size=block_size, max_admit=n_requests,
+                                     max_running=n_requests, max_step_tokens=chunk + n_requests, prefill_chunk=chunk,
+                                     max_seq_len=1024 + new_tokens + block_size))
+    for i in range(reps + 1):
         reqs = [eng.add(p, SamplingParams(max_tokens=new_tokens)) for p in prompts]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -146,10 +150,10 @@ def serve_run(model, cfg, n_requests: int, new_tokens: int, chunk: int, block_si
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         assert all(len(r.out_tokens) == new_tokens for r in reqs)
-        if best is None or dt < best[0]:
+        if i and (best is None or dt < best[0]):
             best = (dt, steps, sum(lens), n_requests * new_tokens)
-        del eng
-        torch.cuda.empty_cache()
+    del eng
+    torch.cuda.empty_cache()
     return best
 
 
@@ -198,10 +202,17 @@ def main() -> int:
                           "config": {"model": SHAPE_NAMES[a.shape], "requests": a.serve, "prompt_tokens": n_prompt, "new_tokens": n_new,
                                      "prompt_len": "uniform 16..1024", "prefill_chunk": 512, "page_size": block}}), flush=True)
         return 0
-    ctx_end = a.ctx + a.steps if a.ctx != 2048 else 4096
-
     steps = a.steps
-    dt, ctx0, ctx1 = decode_run(model, cfg, a.batch, prompt, a.ctx, steps, a.warmup, block, seed=1)
+    whole_run = a.ctx == 2048 and steps >= 2048
+    if a.ctx == 2048 and not whole_run:
+        # a window of the run from 2,048 to 4,096, centred on its mean context (the requests are batch / 2 tokens into
+        # their decoding, on average, when the last is through its prompt)
+        first_ctx = 3072 - steps // 2 - a.warmup - 1 - a.batch
+        window = f"{steps} steps centred on context 3072, the mean of the run from 2048 to 4096"
+    else:
+        first_ctx = a.ctx
+        window = "the whole run" if whole_run else f"{steps} steps from context {a.ctx}"
+    dt, ctx0, ctx1 = decode_run(model, cfg, a.batch, prompt, first_ctx, steps, a.warmup, block, seed=1)
     ms = 1000 * dt / steps
     value = a.batch * steps / dt
     mean_ctx = (ctx0 + ctx1 - 1) / 2
@@ -212,28 +223,30 @@ def main() -> int:
     p_dt = prefill_run(model, cfg, p_tokens, block, portion=a.prefill_portion)
     p_frac = prefill_flops(cfg, p_tokens, 1) / p_dt / PEAK_FLOPS[a.dtype]
 
-    points = {}
+    points, points_frac = {}, {}
     if not a.no_points:
         k = min(steps, 256)
         for b in (1, 64):
             lead = b  # the requests are b / 2 tokens into their decoding, on average, when the last is through its prompt
-            d, _, _ = decode_run(model, cfg, b, prompt, 3072 - k // 2 - a.warmup - 1 - lead, k, a.warmup, block, seed=2 + b)
+            d, c0, c1 = decode_run(model, cfg, b, prompt, 3072 - k // 2 - a.warmup - 1 - lead, k, a.warmup, block, seed=2 + b)
             points[f"decode_b{b}"] = round(b * k / d, 1)
+            nbytes = weight_bytes(cfg, esize) + b * (c0 + c1 - 1) / 2 * kv_bytes_per_token(cfg, esize)
+            points_frac[f"decode_b{b}"] = round(nbytes / (d / k) / 1e9 / HBM_GBPS, 4)
 
     line = {
-        "metric": f"decode tok/s at bs {a.batch}, ctx {a.ctx}->{ctx_end} ({SHAPE_NAMES[a.shape]}, {a.dtype}); prefill tok/s @{p_tokens} tok",
+        "metric": f"decode tok/s at bs {a.batch}, ctx {ctx0:.0f}->{ctx1 - 1:.0f} ({SHAPE_NAMES[a.shape]}, {a.dtype}); prefill tok/s @{p_tokens} tok",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
         "config": {"model": SHAPE_NAMES[a.shape], "layers": shape["num_hidden_layers"], "layers_of_shape": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "global_batch": a.batch, "seq_len": ctx_end, "prompt_len": a.ctx, "ctx_first_step": round(ctx0, 1),
-                   "ctx_last_step": round(ctx1 - 1, 1), "page_size": block, "parallelism": "single GPU", "graphs": True},
+                   "global_batch": a.batch, "seq_len": int(round(ctx1 - 1)), "prompt_len": first_ctx, "ctx_first_step": round(ctx0, 1),
+                   "ctx_last_step": round(ctx1 - 1, 1), "timed": window, "page_size": block, "parallelism": "single GPU", "graphs": True},
         "prefill": {"value": round(p_tokens / p_dt, 1), "tokens": p_tokens, "ms": round(1000 * p_dt, 3), "frac": round(p_frac, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
-        "points": points,
+        "points": points, "points_hbm_frac": points_frac,
     }
     print(json.dumps(line), flush=True)
     return 0

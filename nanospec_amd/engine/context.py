@@ -85,10 +85,15 @@ class StepContext:
 
 
 def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, slots, want_rows, tables: list[np.ndarray],
-               kv_layers: int = 1) -> None:
+               kv_layers: int = 1, pad_tail: int | None = None) -> None:
     """Write one batch into ``host`` (int32, at least layout.total long).  ``starts``/``lens``: first
     position and token count per request; ``tables[g]``: int32 [B, P] block tables; ``kv_layers``: how many layers keep
-    keys and values in pages."""
+    keys and values in pages.
+
+    ``pad_tail`` (batches of a fixed shape, for captured steps): the last request of the batch is a stand-in that owns
+    the last ``pad_tail`` token rows; they are all at position 0 (of a page nobody reads) and no tile covers them.  The
+    layout's tile lists may then be longer than the batch needs: the rest of the prompt-portion tiles hold no tokens, and
+    ``want_rows`` is filled up with row 0."""
     f = layout.fields
     B = layout.B
     lens_a = np.asarray(lens, dtype=np.int32)
@@ -103,15 +108,21 @@ def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, s
     put("token_ids", np.asarray(token_ids, dtype=np.int32))
     req_of = np.repeat(np.arange(B, dtype=np.int32), lens_a)
     put("token_req", req_of)
-    put("positions", np.arange(layout.N, dtype=np.int32) - indptr[req_of] + starts_a[req_of])
+    positions = np.arange(layout.N, dtype=np.int32) - indptr[req_of] + starts_a[req_of]
+    tiled = B if pad_tail is None else B - 1  # requests that the tile lists cover
+    if pad_tail:
+        positions[layout.N - pad_tail :] = 0
+    put("positions", positions)
     put("qo_indptr", indptr)
     put("kv_lens", starts_a + lens_a)
     put("state_slots", np.asarray(slots, dtype=np.int32))
     if layout.R:
-        put("want_rows", np.asarray(want_rows, dtype=np.int32))
+        off, size = f["want_rows"]
+        host[off : off + len(want_rows)] = np.asarray(want_rows, dtype=np.int32)
+        host[off + len(want_rows) : off + size] = 0
     kv = starts_a + lens_a
     if layout.Td:
-        req = np.nonzero(lens_a == 1)[0].astype(np.int32)
+        req = np.nonzero(lens_a[:tiled] == 1)[0].astype(np.int32)
         d = np.zeros((len(req), TILE_INTS), dtype=np.int32)
         d[:, 0], d[:, 2], d[:, 3], d[:, 4] = req, indptr[req], 1, kv[req]
         # keys the decode rows read in this step over all layers: what would have to stay cached until the next step, by
@@ -119,7 +130,8 @@ def fill_batch(host: np.ndarray, layout: BatchLayout, token_ids, starts, lens, s
         d[:, 5] = min(int(kv[req].sum()) * kv_layers, 2**31 - 1)
         put("dtiles", d.reshape(-1))
     if layout.Tc:
-        rows = [(b, t0, indptr[b], n, kv[b], 0, 0, 0) for b, n in enumerate(lens) if n != 1 for t0 in range(0, n, CHUNK_TILE)]
+        rows = [(b, t0, indptr[b], n, kv[b], 0, 0, 0) for b, n in enumerate(lens[:tiled]) if n != 1 for t0 in range(0, n, CHUNK_TILE)]
+        rows += [(B - 1, 0, 0, 0, 0, 0, 0, 0)] * (layout.Tc - len(rows))  # tiles without tokens
         put("ctiles", np.asarray(rows, dtype=np.int32).reshape(-1))
     for g, off in enumerate(layout.table_off):
         host[off : off + B * layout.P] = tables[g].reshape(-1)

@@ -153,7 +153,8 @@ class Engine:
         sampling = [w for w, smp in zip(work, samples) if smp]
         # one uniform per request and step from its own generator (reference: engine/engine.py:283)
         uniforms = [float(torch.rand(1, generator=w.req.gen)) for w in sampling]
-        in_graph = ([w.req.params for w in sampling], uniforms) if len(sampling) == len(work) else None
+        # one per wanted place; with ``profile`` sampling stays a phase of its own, so that its time can be told apart
+        in_graph = ([w.req.params for w in sampling], uniforms) if sampling and not self.config.profile else None
         logits = self.runner.step(entries, device_tokens, sampling=in_graph)
         self._mark("forward")
         for w in work:

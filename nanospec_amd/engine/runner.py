@@ -2,8 +2,9 @@
 
 ``ModelRunner.step`` runs only the tokens it is given, as one batch, from the cache that earlier steps
 left: portions of prompts beside single decoded tokens, cut anywhere.  It reserves pages for the new
-tokens, builds the batch, runs the model and commits the new lengths.  Steps that hold one token per
-request replay a captured HIP graph when the model allows it.
+tokens, builds the batch, runs the model and commits the new lengths.  Steps of one token per request,
+and steps of a few prompt portions of moderate length beside such rows, replay a captured HIP graph of
+a fixed shape when the model allows it; every other step is launched kernel by kernel.
 
 Reference: engine/engine.py:200-252 (rows per request, one forward, hidden states at the last rows)
 and model/llama.py:269-286 (logits only at the rows asked for).  Unlike the reference, prompts and
@@ -21,7 +22,7 @@ from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage
 from ..kernels import ops
 from .arena import Arena
-from .context import BatchLayout, StepContext, count_tiles, fill_batch
+from .context import CHUNK_TILE, BatchLayout, StepContext, count_tiles, fill_batch
 
 # reference: engine/graphs.py:22 (powers of two up to 64).  48 and 96 besides: the products' cost goes by 16 rows at a time
 # between 17 and 128 rows, so 40 requests padded to 64 rows pay for a quarter more than padded to 48.  Above 128 rows
@@ -38,27 +39,44 @@ class StepEntry:
     want: list[int] = field(default_factory=list)  # places among ``tokens`` whose logits are wanted
 
 
-class _DecodeGraph:
-    """One captured decode step for a bucket of ``size`` requests: static batch buffer, fixed arena,
-    logits for every row."""
+# Steps that hold prompt portions beside decode rows are captured too, in fixed shapes: so many rows of one token each (a
+# bucket, or none), so many tokens of prompt portions (padded to a multiple of MIXED_TOKEN_STEP) of at most MIXED_PORTIONS
+# requests.  Launching such a step kernel by kernel costs the host about 0.1 ms a layer, more than the kernels of a small
+# model take.  Longer steps run eagerly: there the GPU's work hides the host's.
+MIXED_PORTIONS = 4
+MIXED_TOKEN_STEP = 64
+MIXED_MAX_TOKENS = 1024
+MAX_GRAPHS = 96  # captured steps kept; the one not used for longest goes first
 
-    def __init__(self, runner: "ModelRunner", size: int, width: int) -> None:
-        self.size, self.width = size, width  # rows; pages per request that its block tables can name
+
+class _StepGraph:
+    """One captured step of a fixed shape: ``rows`` requests that bring one token each and up to ``portions`` requests
+    that bring ``chunk`` tokens together; a static batch buffer, an arena of fixed addresses, logits and samples for
+    ``rows + portions`` wanted places.  What a step does not fill is padding: pad rows and pad tokens belong to the
+    runner's pad request (position 0 of a page nobody reads), tiles without tokens, wanted rows that nobody reads."""
+
+    def __init__(self, runner: "ModelRunner", rows: int, chunk: int, width: int) -> None:
+        self.rows, self.chunk, self.width = rows, chunk, width  # width: pages per request that its block tables can name
+        self.portions = MIXED_PORTIONS if chunk else 0
         n_groups = len(runner.manager.groups)
-        self.layout = BatchLayout(size, size, size, 0, size, n_groups, width, n_patch=size, n_sample=size)
+        self.n_reqs = rows + self.portions + (1 if chunk else 0)  # the last one owns the pad tokens
+        self.n_want = rows + self.portions
+        tiles = chunk // CHUNK_TILE + self.portions if chunk else 0  # every portion may end in a tile that is not full
+        self.layout = BatchLayout(rows + chunk, self.n_reqs, self.n_want, tiles, rows, n_groups, width, n_patch=rows, n_sample=self.n_want)
         dev = runner.device
         self.dev_buf = torch.zeros(self.layout.total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
         self.host_np = self.host.numpy()
         self.arena = Arena(dev)  # grows during the warm-up run, then stays as it is
         self.logits: torch.Tensor | None = None
-        self.sampled = torch.zeros((3, size), dtype=torch.int32, device=dev)  # what the captured sampling kernel writes
+        self.sampled = torch.zeros((3, self.n_want), dtype=torch.int32, device=dev)  # what the captured sampling kernel writes
         self.graph = None
+        self.used = 0
 
     def sample_options(self):
-        """Views of the batch buffer: (temperature, top_p, uniform) float32 and top_k int32, one per row."""
+        """Views of the batch buffer: (temperature, top_p, uniform) float32 and top_k int32, one per wanted place."""
         off, n = self.layout.fields["sample_opts"]
-        opts = self.dev_buf[off : off + n].view(4, self.size)
+        opts = self.dev_buf[off : off + n].view(4, self.n_want)
         f = opts[:3].view(torch.float32)
         return f[0], f[1], f[2], opts[3]
 
@@ -90,7 +108,9 @@ class ModelRunner:
         self._host = torch.zeros(1 << 14, dtype=torch.int32).pin_memory()
         self._dev = torch.zeros(1 << 14, dtype=torch.int32, device=self.device)
         self.use_graphs = bool(use_graphs and model.graph_safe)
-        self._graphs: dict[int, _DecodeGraph] = {}  # by rows; one per bucket, recaptured wider when a request outgrows it
+        # captured steps by (rows of one token, tokens of prompt portions); recaptured wider when a request outgrows one
+        self._graphs: dict[tuple[int, int], _StepGraph] = {}
+        self._graph_uses = 0
         self._pad_ready = False
         self._staged: torch.cuda.Event | None = None
         self.last_used_graph = False
@@ -134,9 +154,9 @@ class ModelRunner:
         those entries is taken from the tensor when the step runs (the id in ``tokens`` is a placeholder), so that a
         step can be enqueued before the step that samples its input has finished.
 
-        ``sampling`` = ([SamplingParams per entry], [uniform number per entry]): if the step replays a captured graph the
-        graph samples too, and ``last_sampled`` is then (int32 [3, bucket] on the GPU, rows that count); otherwise
-        ``last_sampled`` is None and the caller samples from the returned logits."""
+        ``sampling`` = ([SamplingParams per wanted place], [uniform number per wanted place]): if the step replays a
+        captured graph the graph samples too, and ``last_sampled`` is then (int32 [3, places of the graph] on the GPU,
+        places that count); otherwise ``last_sampled`` is None and the caller samples from the returned logits."""
         self.last_sampled = None
         if not entries:
             return None
@@ -171,8 +191,9 @@ class ModelRunner:
         if self._staged is not None:
             self._staged.synchronize()  # the last batch has left the pinned staging buffers
         with torch.cuda.stream(self.stream):
-            if self.use_graphs and all(n == 1 for n in lens) and n_want and self._bucket(len(entries)) is not None:
-                logits = self._step_graph(entries, rcs, starts, device_tokens, sampling)
+            shape = self._graph_shape(lens, n_want) if self.use_graphs else None
+            if shape is not None:
+                logits = self._step_graph(shape, entries, rcs, starts, lens, n_want, device_tokens, sampling)
                 self.last_used_graph = True
             else:
                 logits = self._step_eager(entries, rcs, starts, lens, n_want, device_tokens)
@@ -252,6 +273,22 @@ class ModelRunner:
     def _bucket(self, n: int) -> int | None:
         return next((b for b in GRAPH_BUCKETS if b >= n), None)
 
+    def _graph_shape(self, lens, n_want: int) -> tuple[int, int] | None:
+        """(rows of one token, tokens of prompt portions) of the captured step that takes this batch, or None if it runs
+        eagerly: nothing wanted, more rows than the largest bucket, more or longer portions than a captured step holds."""
+        if not n_want:
+            return None
+        singles = sum(1 for n in lens if n == 1)
+        rows = self._bucket(singles) if singles else 0
+        if rows is None:
+            return None
+        if singles == len(lens):
+            return (rows, 0) if n_want <= rows else None
+        tokens = sum(lens) - singles
+        if len(lens) - singles > MIXED_PORTIONS or tokens > MIXED_MAX_TOKENS or n_want > rows + MIXED_PORTIONS:
+            return None
+        return rows, -(-tokens // MIXED_TOKEN_STEP) * MIXED_TOKEN_STEP
+
     def _ensure_pad(self) -> None:
         if not self._pad_ready:
             self.admit(PAD_REQUEST)  # through admit(): the slot's mirrored block table starts empty
@@ -259,21 +296,38 @@ class ModelRunner:
             self._mirror(self.manager.get(PAD_REQUEST))
             self._pad_ready = True
 
-    def _fill_graph(self, g: _DecodeGraph, entries, rcs, starts, device_tokens=None, sampling=None) -> None:
+    def _fill_graph(self, g: _StepGraph, entries, rcs, starts, lens, device_tokens=None, sampling=None) -> int:
         """Real rows first, then pad rows that read and write the reserved pad page at position 0
-        (reference: engine/graphs.py:115-167)."""
+        (reference: engine/graphs.py:115-167); then the prompt portions and the pad tokens.  -> wanted places filled."""
         pad = self.manager.get(PAD_REQUEST)
-        n_pad = g.size - len(entries)
-        slots = [rc.slot for rc in rcs] + [pad.slot] * n_pad
-        token_ids = [e.tokens[0] for e in entries] + [0] * n_pad
-        st = list(starts) + [0] * n_pad
+        single = [i for i, n in enumerate(lens) if n == 1]
+        multi = [i for i, n in enumerate(lens) if n != 1]
+        n_pad_rows, n_pad_portions = g.rows - len(single), g.portions - len(multi)
+        slots = [rcs[i].slot for i in single] + [pad.slot] * n_pad_rows + [rcs[i].slot for i in multi]
+        token_ids = [entries[i].tokens[0] for i in single] + [0] * n_pad_rows
+        st = [starts[i] for i in single] + [0] * n_pad_rows + [starts[i] for i in multi]
+        ln = [1] * g.rows + [lens[i] for i in multi]
+        first_row = {i: r for r, i in enumerate(single)}
+        at = g.rows
+        for i in multi:
+            first_row[i] = at
+            token_ids += entries[i].tokens
+            at += lens[i]
+        tail = None
+        if g.chunk:
+            tail = g.rows + g.chunk - at
+            slots += [pad.slot] * (n_pad_portions + 1)
+            st += [0] * (n_pad_portions + 1)
+            ln += [0] * n_pad_portions + [tail]
+            token_ids += [0] * tail
+        want_rows = [first_row[i] + w for i, e in enumerate(entries) for w in e.want]
         tables = [t[slots, : g.width] for t in self._tables]
-        fill_batch(g.host_np, g.layout, token_ids, st, [1] * g.size, slots, list(range(g.size)), tables, self._kv_layers)
+        fill_batch(g.host_np, g.layout, token_ids, st, ln, slots, want_rows, tables, self._kv_layers, pad_tail=tail)
         if device_tokens:
-            self._put_patch(g.host_np, g.layout, [e for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
+            self._put_patch(g.host_np, g.layout, [first_row[e] for e, _ in device_tokens[1]], [r for _, r in device_tokens[1]])
         off, n = g.layout.fields["sample_opts"]
-        opts = g.host_np[off : off + n].reshape(4, g.size)
-        opts[:] = 0  # pad rows: temperature 0
+        opts = g.host_np[off : off + n].reshape(4, g.n_want)
+        opts[:] = 0  # places that nobody reads: temperature 0
         if sampling is not None:
             params, uniforms = sampling
             k = len(params)
@@ -289,26 +343,31 @@ class ModelRunner:
         self._staged.record(self.stream)
         if device_tokens:
             self._apply_patch(g.dev_buf, g.layout, device_tokens[0], len(device_tokens[1]))
+        return len(want_rows)
 
     GRAPH_MIN_WIDTH = 16  # pages per request that the narrowest captured step's block tables hold
 
-    def _graph_for(self, size: int, pages: int) -> _DecodeGraph:
-        """The captured step of ``size`` rows, its block tables wide enough for ``pages`` pages per request.  Tables are as
-        wide as the longest request has needed so far, rounded up to a power of two (every replay fills and copies rows x
-        width ints), so a bucket is captured again, twice as wide, when a request outgrows it."""
-        g = self._graphs.get(size)
-        if g is not None and g.width >= pages:
-            return g
-        width = max(self.GRAPH_MIN_WIDTH, 1 << (pages - 1).bit_length())
-        width = min(width, self.table_width)
-        if g is not None:
-            self.stream.synchronize()  # the narrower graph may still be running
-            del self._graphs[size]
-        return self._capture(size, width)
+    def _graph_for(self, shape: tuple[int, int], pages: int) -> _StepGraph:
+        """The captured step of this shape, its block tables wide enough for ``pages`` pages per request.  Tables are as
+        wide as the longest request has needed so far, rounded up to a power of two (every replay fills and copies
+        requests x width ints), so a shape is captured again, twice as wide, when a request outgrows it."""
+        g = self._graphs.get(shape)
+        if g is None or g.width < pages:
+            width = max(self.GRAPH_MIN_WIDTH, 1 << (pages - 1).bit_length())
+            width = min(width, self.table_width)
+            if g is not None or len(self._graphs) >= MAX_GRAPHS:
+                self.stream.synchronize()  # a graph that is dropped may still be running
+                self._graphs.pop(shape, None)
+                if len(self._graphs) >= MAX_GRAPHS:
+                    del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].used)]
+            g = self._capture(shape, width)
+        self._graph_uses += 1
+        g.used = self._graph_uses
+        return g
 
-    def _capture(self, size: int, width: int) -> _DecodeGraph:
-        g = _DecodeGraph(self, size, width)
-        self._fill_graph(g, [], [], [])
+    def _capture(self, shape: tuple[int, int], width: int) -> _StepGraph:
+        g = _StepGraph(self, shape[0], shape[1], width)
+        self._fill_graph(g, [], [], [], [])
         ctx = g.context(self)
 
         def run():
@@ -327,26 +386,24 @@ class ModelRunner:
         with graph:
             g.logits = run()
         g.graph = graph
-        self._graphs[size] = g
+        self._graphs[shape] = g
         return g
 
-    def _step_graph(self, entries, rcs, starts, device_tokens=None, sampling=None):
+    def _step_graph(self, shape, entries, rcs, starts, lens, n_want, device_tokens=None, sampling=None):
         self._ensure_pad()
-        size = self._bucket(len(entries))
-        max_kv = max(starts) + 1
+        max_kv = max(s + n for s, n in zip(starts, lens))
         pages = -(-max_kv // self.page_size)
         if pages > self.table_width:
             raise ValueError(f"a request needs {pages} pages; block tables hold {self.table_width}")
         self.model.check_positions(max_kv - 1)
-        g = self._graph_for(size, pages)
-        self._fill_graph(g, entries, rcs, starts, device_tokens, sampling)
+        g = self._graph_for(shape, pages)
+        if sampling is not None and len(sampling[0]) != n_want:
+            sampling = None  # the caller samples from the logits
+        self._fill_graph(g, entries, rcs, starts, lens, device_tokens, sampling)
         g.graph.launch()
-        if sampling is not None and all(e.want for e in entries):
-            self.last_sampled = (g.sampled, len(entries))
-        rows = [i for i, e in enumerate(entries) if e.want]
-        if len(rows) == len(entries):
-            return g.logits[: len(entries)]
-        return g.logits[rows]
+        if sampling is not None:
+            self.last_sampled = (g.sampled, n_want)
+        return g.logits[:n_want]
 
     def synchronize(self) -> None:
         self.stream.synchronize()

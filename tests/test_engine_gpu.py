@@ -320,7 +320,7 @@ def test_many_requests_decode_through_one_graph(tiny_folders, n_requests, bucket
     new = 5
     reqs, _, eng = run_engine(model, prompts, [SamplingParams(max_tokens=new)] * n_requests, num_blocks=900, block_size=8,
                               max_admit=n_requests, max_running=n_requests)
-    assert bucket in eng.runner._graphs, f"the {n_requests} rows did not replay the graph of {bucket}"
+    assert (bucket, 0) in eng.runner._graphs, f"the {n_requests} rows did not replay the graph of {bucket}"
     for i, (p, r) in enumerate(zip(prompts, reqs)):
         assert len(r.out_tokens) == new
         rows = pl.logits_of_sequence(w, cfg, p + r.out_tokens[:-1], torch.bfloat16)[len(p) - 1 :]

@@ -94,6 +94,8 @@ def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, link_
         rep.scattered = 0
     for step, w in zip(steps, where):
         out = rep.step(step["entries"], step["end"])
+        if rep.runner.last_used_graph and any(len(e["tokens"]) > 1 for e in step["entries"]):
+            rep.mixed_graph_steps = getattr(rep, "mixed_graph_steps", 0) + 1
         if churned:
             for e in step["entries"]:
                 if e["id"] in rep.manager:
@@ -166,6 +168,34 @@ def test_long_decoding_from_the_first_token(tiny_folders, name, dtype):
     replay(model, steps, where, ref, dtype, 512, page)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_steps_replay_captured_steps_of_fixed_shapes(tiny_folders, name, dtype):
+    """Steps of a few prompt portions beside decode rows replay captured steps whose shapes are padded (pad rows, pad
+    tokens, tiles without tokens, wanted places nobody reads); the same trace without graphs gives the same logits, and
+    both are the plain implementation's.  Few logits are wanted per step here, as in generation: a captured step has room
+    for one per row and one per portion."""
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, dtype)
+    model = engine_model(folder, name, dtype)
+    steps, where, peak = traces.mixed(seqs, seed=11)
+    thin_steps, thin_where = [], []
+    for step, w in zip(steps, where):  # keep the last wanted place of every entry only
+        entries, at, kept = [], 0, []
+        for e in step["entries"]:
+            n = len(e["want"])
+            entries.append(dict(e, want=e["want"][-1:]))
+            kept += w[at + n - 1 : at + n]
+            at += n
+        thin_steps.append(dict(step, entries=entries))
+        thin_where.append(kept)
+    rep = replay(model, thin_steps, thin_where, ref, dtype, peak, page, graphs=True)
+    assert getattr(rep, "mixed_graph_steps", 0) >= 10, "the mixed steps were meant to replay captured steps"
+    assert any(chunk for _, chunk in rep.runner._graphs)
+    replay(model, thin_steps, thin_where, ref, dtype, peak, page, graphs=False)
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_graph_and_eager_decode_agree(tiny_folders, name):
     folder, page = tiny_folders[name], TINY[name]["page"]
@@ -211,7 +241,7 @@ def test_every_graph_bucket_against_plain(tiny_folders, n_requests, bucket):
     for d in range(decoded, 0, -1):
         entries = [{"id": r, "tokens": [seqs[r][-d]], "want": [0]} for r in ids]
         out = rep.step(entries, ids if d == 1 else [])
-        assert rep.runner.last_used_graph and bucket in rep.runner._graphs
+        assert rep.runner.last_used_graph and (bucket, 0) in rep.runner._graphs
         want = torch.stack([ref[r][len(seqs[r]) - d] for r in ids])
         check(out, want, torch.bfloat16, f"{n_requests} requests, {d} tokens before their end")
     rep.manager.check()
@@ -470,7 +500,7 @@ def test_benchmark_shape_slice_matches_plain(llama_8b_slice, dtype):
             at[r] += n
         out = rep.step(entries, [])
         if graph is not None:
-            assert rep.runner.last_used_graph and graph in rep.runner._graphs
+            assert rep.runner.last_used_graph and (graph, 0) in rep.runner._graphs
         if places:
             check(out, plain_rows(places), dtype, str([(r, n) for r, n, _ in parts][:4]))
         else:
