@@ -416,6 +416,85 @@ extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions,
   return ns_launch_status();
 }
 
+// The same for a stacked q/k/v product whose K was cut into ranges that are not added up yet (17 to 128 rows through
+// ns_gemm_wide_bf16 with `defer`), from the weight tiled in the row order of the fused few-row kernel (gemm_bf16.hip,
+// EPI_ROPE_KV): a tile of 16 columns of the product is, in the rotary part of a q or k head, 8 channels j and their
+// partners j + rot/2, elsewhere 16 consecutive channels.  One pass adds the ranges in order, rotates the 32-bit sums,
+// rounds once, and writes q to the attention input, k to its K page slot and v to the transposed V page.
+//   partial[s][m][c]: range s, token m, column c of the product (columns in the tiled row order)
+//   thread <-> (token, tile of 16 columns, pair p of columns p and p + 8)
+__global__ __launch_bounds__(256) void rope_kv_partial_kernel(bf16_t* __restrict__ q_out, int q_stride, const float* __restrict__ partial,
+                                                              int ksplit, int M, int N, const int* __restrict__ positions,
+                                                              const int* __restrict__ token_req, const int* __restrict__ block_table,
+                                                              int table_stride, const float* __restrict__ inv_freq,
+                                                              bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int heads,
+                                                              int kv_heads, int hd, int rot, int page_size, int write_kv) {
+  const int m = blockIdx.x;
+  const int u = blockIdx.y * blockDim.x + threadIdx.x;  // (tile, pair)
+  const int tiles_per_head = hd / 16;
+  const int tile = u >> 3, p = u & 7;
+  if (tile >= (heads + 2 * kv_heads) * tiles_per_head) return;
+  const int gh = tile / tiles_per_head, jt = tile - gh * tiles_per_head;  // head among [q heads | k heads | v heads]
+  const bool is_q = gh < heads, is_v = gh >= heads + kv_heads;
+  if (!is_q && !write_kv) return;
+  const int rot_tiles = is_v ? 0 : rot / 16;
+  const bool rotary = jt < rot_tiles;
+  const size_t plane = (size_t)M * N;
+  const float* src = partial + (size_t)m * N + tile * 16 + p;
+  float x1 = 0.f, x2 = 0.f;
+  for (int s = 0; s < ksplit; ++s) {
+    x1 += src[s * plane];
+    x2 += src[s * plane + 8];
+  }
+  const int pos = positions[m];
+  int d1, d2;
+  if (rotary) {
+    const int j = jt * 8 + p;
+    const float ang = (float)pos * inv_freq[j];
+    const float c = cosf(ang), sn = sinf(ang);
+    const float a = x1, b = x2;
+    x1 = a * c - b * sn;
+    x2 = b * c + a * sn;
+    d1 = j;
+    d2 = j + rot / 2;
+  } else {
+    d1 = (is_v ? 0 : rot) + (jt - rot_tiles) * 16 + p;
+    d2 = d1 + 8;
+  }
+  if (is_q) {
+    bf16_t* o = q_out + (size_t)m * q_stride + gh * hd;
+    o[d1] = (bf16_t)x1;
+    o[d2] = (bf16_t)x2;
+    return;
+  }
+  const int page = block_table[(size_t)token_req[m] * table_stride + pos / page_size];
+  const int off = pos % page_size;
+  if (!is_v) {
+    bf16_t* kd = k_cache + (((size_t)page * kv_heads + (gh - heads)) * page_size + off) * hd;
+    kd[d1] = (bf16_t)x1;
+    kd[d2] = (bf16_t)x2;
+  } else {
+    bf16_t* vd = v_cache + (((size_t)page * kv_heads + (gh - heads - kv_heads)) * hd) * page_size + off;
+    vd[(size_t)d1 * page_size] = (bf16_t)x1;
+    vd[(size_t)d2 * page_size] = (bf16_t)x2;
+  }
+}
+
+extern "C" int ns_rope_kv_partial(void* q_out, int q_stride, const float* partial, int ksplit, int M, int N, const int* positions,
+                                  const int* token_req, const int* block_table, int table_stride, const float* inv_freq,
+                                  void* k_cache, void* v_cache, int heads, int kv_heads, int hd, int rot, int page_size, int write_kv,
+                                  hipStream_t stream) {
+  if (M <= 0 || M > 65535 || ksplit < 1 || heads <= 0 || kv_heads <= 0 || hd <= 0 || (hd & 15) || rot < 0 || rot > hd || (rot & 15) ||
+      page_size <= 0 || N != (heads + 2 * kv_heads) * hd || q_stride < heads * hd)
+    return NS_ERR_BAD_ARG;
+  const int units = N / 2;  // pairs of columns per token
+  dim3 grid(M, (units + 255) / 256);
+  rope_kv_partial_kernel<<<grid, 256, 0, stream>>>((bf16_t*)q_out, q_stride, partial, ksplit, M, N, positions, token_req, block_table,
+                                                   table_stride, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, rot,
+                                                   page_size, write_kv);
+  return ns_launch_status();
+}
+
 // ------------------------------------------------------------------------------------------------
 // out[n, i] = silu(gu[n, i]) * gu[n, inter + i]                 (reference: model/llama.py:195)
 // ------------------------------------------------------------------------------------------------

@@ -515,6 +515,32 @@ def linear_qkv_rope(x: "torch.Tensor | PreNormed", w: TiledWeight, q_out: torch.
                                               _stream()), "linear_qkv_rope")
 
 
+def rope_kv_from_partial(p: PartialSums, q_out: torch.Tensor, positions, token_req, block_table, inv_freq, k_cache, v_cache,
+                         heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
+    """Rotation and cache write for a stacked q/k/v product whose K ranges are not added up yet (``linear_wide(...,
+    defer=True)`` from a weight tiled in ``qkv_rope_row_order``): one pass adds the ranges, rotates, and writes q into
+    ``q_out`` [rows, >= heads * head_dim], k into its K page slot and v into the transposed V page."""
+    _gpu(p.ws, q_out, positions, token_req, block_table, inv_freq, k_cache, v_cache)
+    m = p.rows
+    if p.dtype != torch.bfloat16 or head_dim % 16 or rotary_dim % 16 or p.n != (heads + 2 * kv_heads) * head_dim:
+        raise KernelRefused("rope_kv_from_partial takes a bfloat16 product of heads + 2 kv_heads heads, head and rotary sizes multiples of 16")
+    if q_out.dtype != torch.bfloat16 or q_out.shape[0] != m or q_out.shape[1] < heads * head_dim or q_out.stride(1) != 1:
+        raise KernelRefused("rope_kv_from_partial: q_out must be bfloat16 [rows, >= heads * head_dim]")
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
+    page = k_cache.shape[2]
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+            or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("rope_kv_from_partial: cache pages do not fit heads, head size or dtype")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2) or positions.numel() != m or token_req.numel() != m:
+        raise KernelRefused("rope_kv_from_partial: positions, token_req are per row; inv_freq holds rotary_dim / 2 float32 values")
+    if p.ws.dtype != torch.float32 or p.ws.numel() < p.ksplit * m * p.n:
+        raise KernelRefused("rope_kv_from_partial: the partial sums are too few")
+    _check(build.core().ns_rope_kv_partial(_ptr(q_out), c_int(q_out.stride(0)), _ptr(p.ws), c_int(p.ksplit), c_int(m), c_int(p.n),
+                                           _ptr(positions), _ptr(token_req), _ptr(block_table), c_int(block_table.stride(0)),
+                                           _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(heads), c_int(kv_heads), c_int(head_dim),
+                                           c_int(rotary_dim), c_int(page), c_int(1 if write_kv else 0), _stream()), "rope_kv_from_partial")
+
+
 # ------------------------------------------------------------------------------------------------ attention
 
 

@@ -153,6 +153,16 @@ class Attention:
         if self.wqkv_rope is not None and n <= 16 and ops.tiled_takes(x.x if isinstance(x, ops.PreNormed) else x, s.hidden):
             ops.linear_qkv_rope(x, self.wqkv_rope, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v,
                                 s.heads, s.kv_heads, s.head_dim, pos.rotary_dim, write_kv=owns_cache)
+        elif (self.wqkv_rope is not None and n <= ops.WIDE_TALL_ROWS and not isinstance(x, ops.PreNormed) and ops.tiled_takes(x[:1], s.hidden)
+              and ops.wide_plan(self.wqkv_rope.n, s.hidden, n)[0] > 1):
+            # 17 to 128 rows: the product streams the same tiled matrix with K cut into ranges, and the kernel that adds the
+            # ranges rotates and writes the cache in the same pass (the library's product and a rotation kernel otherwise)
+            ksplit, nt = ops.wide_plan(self.wqkv_rope.n, s.hidden, n)
+            ksplit = min(ksplit, 4)  # (the joining kernel reads every range: more of them cost it what they gain the product)
+            ws = ctx.arena.take((ksplit * n * self.wqkv_rope.n,), torch.float32)
+            part = ops.linear_wide(x, self.wqkv_rope, workspace=ws, ksplit=ksplit, nt=nt, defer=True)
+            ops.rope_kv_from_partial(part, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
+                                     s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         else:
             self.wqkv(x, out=qkv, arena=ctx.arena)
             ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,

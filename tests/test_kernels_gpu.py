@@ -266,6 +266,53 @@ def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, pa
         assert ulps_of_row_max(v[pg, :, :, off].cpu().reshape(1, -1), v0[t].reshape(1, -1)).max() <= 1.0
 
 
+@pytest.mark.parametrize("rows", [17, 40, 64, 100, 128])
+@pytest.mark.parametrize("heads,kvh,hd,rot,page,hidden,ksplit", [(6, 3, 32, 32, 4, 384, 3), (4, 1, 48, 16, 8, 520, 2), (8, 2, 128, 128, 16, 1024, 4),
+                                                                 (2, 2, 16, 0, 4, 256, 2)])
+def test_qkv_product_in_ranges_joined_by_the_rotation_kernel(rows, heads, kvh, hd, rot, page, hidden, ksplit):
+    """17 to 128 rows: the stacked product with K cut into ranges from the matrix tiled in the few-row kernel's row order,
+    and one kernel that adds the ranges, rotates q and k and writes k and v into their pages; against the plain product
+    followed by the plain rotation.  Requests of several tokens and of one, pages scattered."""
+    ops = _ops()
+    torch.manual_seed(hd + rot + rows)
+    lens = [rows - 9, 1, 5, 1, 2] if rows > 20 else [rows - 4, 1, 3]
+    starts = [3, 0, 9, 30, 1][: len(lens)]
+    n = sum(lens)
+    assert n == rows
+    table = scattered_tables([s + l for s, l in zip(starts, lens)], page, 64, seed=2).to(DEV)
+    positions = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    w = (torch.randn((heads + 2 * kvh) * hd, hidden) * 0.3).to(torch.bfloat16)
+    x = torch.randn(n, hidden).to(torch.bfloat16)
+    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot))
+    q_out = torch.zeros(n, (heads + 2 * kvh) * hd, dtype=torch.bfloat16, device=DEV)
+    k, v = make_cache(64, page, kvh, hd, torch.bfloat16)
+    inv = pl.inverse_frequencies(rot, 10000.0, None) if rot else torch.zeros(1)
+    part = ops.linear_wide(x.to(DEV), wt, ksplit=ksplit, nt=1, defer=True)
+    assert isinstance(part, ops.PartialSums) and part.ksplit == ksplit
+    ops.rope_kv_from_partial(part, q_out, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot)
+    full = x.float() @ w.float().T  # 32-bit sums: the kernel rotates before it rounds
+    q0 = full[:, : heads * hd].view(n, heads, hd)
+    k0 = full[:, heads * hd : (heads + kvh) * hd].view(n, kvh, hd)
+    v0 = full[:, (heads + kvh) * hd :].view(n, kvh, hd)
+    if rot:
+        cos, sin = pl.rotation_tables(positions.cpu(), inv)
+        q0 = torch.cat([pl.rotate(q0[..., :rot], cos, sin), q0[..., rot:]], -1)
+        k0 = torch.cat([pl.rotate(k0[..., :rot], cos, sin), k0[..., rot:]], -1)
+    assert ulps_of_row_max(q_out[:, : heads * hd].cpu(), q0.reshape(n, -1)).max() <= 1.0
+    assert torch.count_nonzero(q_out[:, heads * hd :]) == 0  # only q goes to the attention input
+    for t in range(n):
+        b, p = int(token_req[t]), int(positions[t])
+        pg, off = int(table[b, p // page]), p % page
+        assert ulps_of_row_max(k[pg, :, off].cpu().reshape(1, -1), k0[t].reshape(1, -1)).max() <= 1.0
+        assert ulps_of_row_max(v[pg, :, :, off].cpu().reshape(1, -1), v0[t].reshape(1, -1)).max() <= 1.0
+    # without the cache write only q is produced
+    k2, v2 = make_cache(64, page, kvh, hd, torch.bfloat16)
+    before = (k2.clone(), v2.clone())
+    ops.rope_kv_from_partial(part, q_out, positions, token_req, table, inv.to(DEV), k2, v2, heads, kvh, hd, rot, write_kv=False)
+    assert torch.equal(k2, before[0]) and torch.equal(v2, before[1])
+
+
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("hidden,inner", [(136, 264), (4096, 1024), (64, 8)])
 def test_product_that_updates_the_residual_and_feeds_the_next_norm(m, hidden, inner):
