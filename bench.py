@@ -7,8 +7,10 @@ step function, captured graphs, sampling).  The benchmark decodes from context 2
 linearly with the context, so K timed steps (after W untimed ones) are taken as a window centred on context 3,072,
 the mean of 2,048..4,096, and stand for the whole run; with K >= 2,048 the whole run is timed (prompts of 2,048
 random token ids, then 2,048 decode steps).  ``metric`` and ``config`` name the contexts that were timed.  ``points``
-holds the same at batch 1 and 64 (windows of at most 256 steps) and ``points_hbm_frac`` their fractions of the
-memory roofline.  ``prefill`` is one step of 2,048 prompt tokens of one request; ``roofline`` is the bytes a decode
+holds the same at batch 1 and 64 (windows of at most 256 steps), and the new tokens per second of 32 requests served by
+continuous batching at the Llama-3.2-1B shape (prompts of 16 to 1,024 tokens in portions of 512, 128 new tokens each);
+``points_roofline_frac`` holds their fractions of the memory roofline (for the serving run: of what memory and matrix units
+need together).  ``prefill`` is one step of 2,048 prompt tokens of one request; ``roofline`` is the bytes a decode
 step must read (every weight once, the cache of the live requests) over its time, against 8 TB/s.
 """
 
@@ -124,7 +126,7 @@ def prefill_run(model, cfg, n_tokens: int, block_size: int, reps: int = 3, porti
 def serve_run(model, cfg, n_requests: int, new_tokens: int, chunk: int, block_size: int, seed: int = 0, reps: int = 2):
     """Continuous batching with chunked prefill: ``n_requests`` arrive at once with prompts of 16 to 1,024 uniform-random
     token ids and generate ``new_tokens`` each; prompts are taken in portions of at most ``chunk`` tokens beside the decoding
-    of the requests that are through theirs.  -> (seconds of the best pass, steps, prompt tokens, new tokens)."""
+    of the requests that are through theirs.  -> (seconds of the best pass, steps, prompt lengths, new tokens)."""
     import torch
 
     from nanospec_amd import Engine, EngineConfig, SamplingParams
@@ -151,10 +153,19 @@ def serve_run(model, cfg, n_requests: int, new_tokens: int, chunk: int, block_si
         dt = time.perf_counter() - t0
         assert all(len(r.out_tokens) == new_tokens for r in reqs)
         if i and (best is None or dt < best[0]):
-            best = (dt, steps, sum(lens), n_requests * new_tokens)
+            best = (dt, steps, lens, n_requests * new_tokens)
     del eng
     torch.cuda.empty_cache()
     return best
+
+
+def serve_ideal_seconds(cfg, esize: int, lens, new_tokens: int, steps: int, dtype: str) -> float:
+    """What the serve workload needs at the least: every step reads the weights once, every decoded token the keys and
+    values of its context, both at the memory's peak rate; and the arithmetic of the prompts at the matrix units' peak."""
+    nbytes = steps * weight_bytes(cfg, esize)
+    nbytes += sum((n + t) * kv_bytes_per_token(cfg, esize) for n in lens for t in range(new_tokens))
+    flops = sum(prefill_flops(cfg, n, 1) for n in lens)
+    return nbytes / (HBM_GBPS * 1e9) + flops / PEAK_FLOPS[dtype]
 
 
 def main() -> int:
@@ -194,10 +205,15 @@ def main() -> int:
     model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
     block, prompt = 16, 2048
     if a.serve:
-        dt, n_steps, n_prompt, n_new = serve_run(model, cfg, a.serve, 128, 512, block)
+        dt, n_steps, lens, n_new = serve_run(model, cfg, a.serve, 128, 512, block)
+        n_prompt = sum(lens)
+        frac = serve_ideal_seconds(cfg, esize, lens, 128, n_steps, a.dtype) / dt
         print(json.dumps({"metric": f"continuous batching with chunked prefill of 512 ({SHAPE_NAMES[a.shape]}, {a.dtype}): new tok/s",
                           "value": round(n_new / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": n_steps, "seconds": round(dt, 4),
                           "all_tokens_per_s": round((n_prompt + n_new) / dt, 1), "higher_is_better": True, "dtype": a.dtype,
+                          "roofline": {"bound": "hbm + matrix units", "frac": round(frac, 4),
+                                       "what": "seconds that the weights of every step, the keys and values of every decoded token (at 8 TB/s) "
+                                               "and the prompts' arithmetic (at the matrix units' peak) need at the least, over the seconds measured"},
                           "data": "synthetic: random weights N(0,0.02), uniform random token ids",
                           "config": {"model": SHAPE_NAMES[a.shape], "requests": a.serve, "prompt_tokens": n_prompt, "new_tokens": n_new,
                                      "prompt_len": "uniform 16..1024", "prefill_chunk": 512, "page_size": block}}), flush=True)
@@ -233,6 +249,20 @@ def main() -> int:
             nbytes = weight_bytes(cfg, esize) + b * (c0 + c1 - 1) / 2 * kv_bytes_per_token(cfg, esize)
             points_frac[f"decode_b{b}"] = round(nbytes / (d / k) / 1e9 / HBM_GBPS, 4)
 
+    if not a.no_points and a.shape == "8b" and not a.layers:
+        # BASELINE's fourth configuration beside the headline: 32 requests through the Llama-3.2-1B shape, continuous batching
+        # with prompts in portions of 512
+        del model
+        torch.cuda.empty_cache()
+        small = dict(SHAPES["1b"])
+        cfg1 = LlamaConfig.from_hf(dict(model_type="llama", **{k: v for k, v in small.items() if k != "rope_scaling"},
+                                        rope_scaling=dict(rope_type="llama3", **small["rope_scaling"])))
+        model1 = random_model(cfg1, seed=0, dtype=dtype, on_device=True)
+        s_dt, s_steps, s_lens, s_new = serve_run(model1, cfg1, 32, 128, 512, block)
+        points["serve_1b_32req_new_tok_s"] = round(s_new / s_dt, 1)
+        points_frac["serve_1b_32req_new_tok_s"] = round(serve_ideal_seconds(cfg1, esize, s_lens, 128, s_steps, a.dtype) / s_dt, 4)
+        del model1
+
     line = {
         "metric": f"decode tok/s at bs {a.batch}, ctx {ctx0:.0f}->{ctx1 - 1:.0f} ({SHAPE_NAMES[a.shape]}, {a.dtype}); prefill tok/s @{p_tokens} tok",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": a.warmup,
@@ -246,7 +276,7 @@ def main() -> int:
         "prefill": {"value": round(p_tokens / p_dt, 1), "tokens": p_tokens, "ms": round(1000 * p_dt, 3), "frac": round(p_frac, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
-        "points": points, "points_hbm_frac": points_frac,
+        "points": points, "points_roofline_frac": points_frac,
     }
     print(json.dumps(line), flush=True)
     return 0
