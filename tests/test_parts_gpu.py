@@ -518,3 +518,109 @@ def test_toy_block_and_other_tensor_names(dtype):
             assert ulps_of_row_max(out.cpu(), want).max() <= 8, entries
     with pytest.raises(ValueError):  # the block's mixer bounds the positions, and the model asks the block
         rep.step([{"id": "c", "tokens": list(range(97)), "want": []}], [])
+
+
+# ------------------------------------------------------- layers that keep a window of keys beside layers that keep all
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_windowed_layers_give_pages_back_while_requests_run(dtype):
+    """One layer sees every earlier key, two see the last ten: two groups of pages.  The windowed group's pool holds far
+    fewer pages than the requests have positions, so pages that a window has passed are given back while the request
+    runs and handed out again, to the same request and to others; block tables then hold released entries, which the
+    kernels must never follow.  Against plain attention over the whole sequences with the window as a mask."""
+    import math
+
+    from nanospec_amd.cache.manager import RELEASED, CacheManager
+    from nanospec_amd.cache.storage import CacheStorage, plan_groups
+    from nanospec_amd.config.spec import AttentionSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
+    from nanospec_amd.engine.runner import ModelRunner, StepEntry
+    from nanospec_amd.parts import DecoderModel
+    from nanospec_amd.weights import DictSource, random_tensors
+
+    hidden, vocab, hd, page, window = 64, 83, 16, 4, 10
+    norm = RMSNormSpec(hidden, 1e-5)
+    ffn = SwiGLUSpec(hidden, 96)
+    full = AttentionSpec(hidden, 4, 2, hd, RopeSpec(hd, 1e4), 1 / math.sqrt(hd))
+    near = AttentionSpec(hidden, 4, 1, hd, RopeSpec(hd, 1e4), 1 / math.sqrt(hd), window=window)
+    layers = tuple(llama_block(f"model.layers.{i}.", norm, a, norm, ffn) for i, a in enumerate((full, near, near)))
+    spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers, tuple(LayerCall(i) for i in range(3)), norm, "model.norm.weight",
+                     "lm_head.weight", True)
+    net = DecoderModel(spec)
+    w = {k: (v * (5.0 if "proj" in k else 1.0)).to(dtype) for k, v in random_tensors(net.wanted(), seed=31, skip={"lm_head.weight"}).items()}
+    model = net.load(DictSource(w), dtype, DEV)
+    specs, _, _ = plan_groups(model.cache_needs)
+    assert [(s.name, s.window) for s in specs] == [("kv2x16", 0), ("kv1x16w10", window)]
+    lengths = {"a": 61, "b": 47, "c": 52}
+    pages = [sum(-(-n // page) for n in lengths.values()) + 2, 14]  # all keys of all requests; 14 pages for the windows
+    manager = CacheManager(specs, pages, page, 8)
+    storage = CacheStorage(model, pages, page, 8, dtype, model.device)
+    runner = ModelRunner(model, manager, storage, 8, max(pages))
+
+    g = torch.Generator().manual_seed(12)
+    seqs = {r: torch.randint(0, vocab, (n,), generator=g).tolist() for r, n in lengths.items()}
+
+    def plain(tokens):
+        t = len(tokens)
+        x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        cos, sin = pl.rotation_tables(torch.arange(t), pl.inverse_frequencies(hd, 1e4, None))
+        for i, (kvh, win) in enumerate(((2, 0), (1, window), (1, window))):
+            p = f"model.layers.{i}."
+            h = pl.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+            q = pl.rotate(pl.linear(h, w[p + "self_attn.q_proj.weight"]).view(t, 4, hd), cos, sin)
+            k = pl.rotate(pl.linear(h, w[p + "self_attn.k_proj.weight"]).view(t, kvh, hd), cos, sin)
+            v = pl.linear(h, w[p + "self_attn.v_proj.weight"]).view(t, kvh, hd)
+            if win:
+                a = torch.cat([pl.causal_attention(q[j : j + 1], k[max(0, j - win + 1) : j + 1], v[max(0, j - win + 1) : j + 1],
+                                                   first_query=min(j, win - 1)) for j in range(t)])
+            else:
+                a = pl.causal_attention(q, k, v)
+            x = pl.residual_add(x, pl.linear(a.reshape(t, -1), w[p + "self_attn.o_proj.weight"]))
+            h = pl.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+            x = pl.residual_add(x, pl.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"]))
+        return pl.rms_norm(x, w["model.norm.weight"], 1e-5).float() @ w["model.embed_tokens.weight"].float().T
+
+    refs = {r: plain(t) for r, t in seqs.items()}
+    at = {r: 0 for r in seqs}
+    granted = {}  # page of the windowed group -> the (request, table index) pairs it has served
+    released_seen = 0
+    import random
+
+    rng = random.Random(3)
+    for r in seqs:
+        runner.admit(r)
+    step_no = 0
+    while any(at[r] < lengths[r] for r in seqs):
+        entries, places = [], []
+        for r in seqs:
+            left = lengths[r] - at[r]
+            if not left or rng.random() < 0.15:
+                continue
+            n = 1 if rng.random() < 0.5 else min(left, rng.choice((2, 3, 4)))  # never more than a page beyond the window
+            entries.append(StepEntry(r, seqs[r][at[r] : at[r] + n], list(range(n))))
+            places += [(r, at[r] + i) for i in range(n)]
+            at[r] += n
+        if not entries:
+            continue
+        out = runner.step(entries).cpu()
+        want = torch.stack([refs[r][p] for r, p in places])
+        if dtype == torch.float32:
+            err = ((out - want).abs().amax(-1) / want.abs().amax(-1)).max()
+            assert err < 1e-4, (step_no, float(err))
+        else:
+            assert ulps_of_row_max(out, want).max() <= 8, step_no
+        manager.check()
+        for r in seqs:
+            table = manager.get(r).tables[1]
+            released_seen += sum(1 for p in table if p == RELEASED)
+            assert manager.get(r).held[1] <= -(-window // page) + 2
+            for i, p in enumerate(table):
+                if p != RELEASED:
+                    granted.setdefault(p, set()).add((r, i))
+        step_no += 1
+    assert released_seen > 100, "the windows were meant to give pages back"
+    assert sum(1 for uses in granted.values() if len(uses) > 1) >= 10, "pages of the windowed group were meant to be used again"
+    assert sum(lengths.values()) > 2 * pages[1] * page  # the windowed pool holds less than half of what was written through it
+    for r in seqs:
+        runner.release(r)
+    manager.check()
