@@ -706,25 +706,10 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
           o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
         }
       };
-      if constexpr (SETS == 2) {
-        // both columns' weights first, then every fragment of the values is read from LDS once and serves both columns
-        // (a third fewer LDS reads per block: 12% faster for a 2,048-token prompt, whose time is its longest chain of blocks)
-        soften(0);
-        soften(1);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
-          o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[0], o[0][dt], 0, 0, 0);
-          o[1][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[1], o[1][dt], 0, 0, 0);
-        }
-      } else {
-        // one set of waves per workgroup, two workgroups to a compute unit out of step with each other: here the order that
-        // lets one column's matrix instructions run under the other's soft-max is the faster one (2 to 3% at 32k keys)
-        soften(0);
-        weigh(0);
-        soften(1);
-        weigh(1);
-      }
+      soften(0);
+      weigh(0);
+      soften(1);
+      weigh(1);
     };
 
     // Before round it: block kb0 + it lies in LDS buffer it & 1, block kb0 + it + 1 is on its way into register set
