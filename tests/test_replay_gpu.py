@@ -196,6 +196,44 @@ def test_mixed_steps_replay_captured_steps_of_fixed_shapes(tiny_folders, name, d
     replay(model, thin_steps, thin_where, ref, dtype, peak, page, graphs=False)
 
 
+def test_captured_steps_are_dropped_and_captured_again(tiny_folders, monkeypatch):
+    """Room for three captured steps only, and block tables that start two pages wide: steps are captured, dropped (the one
+    unused for longest first) and captured again, and captured again wider whenever a request outgrows them; the logits
+    stay the plain implementation's throughout."""
+    from nanospec_amd.engine import runner as runner_mod
+
+    name = "A"
+    folder, page = tiny_folders[name], TINY[name]["page"]
+    seqs = sequences(name)
+    ref = plain_logits(folder, name, torch.bfloat16)
+    model = engine_model(folder, name, torch.bfloat16)
+    monkeypatch.setattr(runner_mod, "MAX_GRAPHS", 3)
+    monkeypatch.setattr(runner_mod.ModelRunner, "GRAPH_MIN_WIDTH", 2)
+    captures = []
+    real = runner_mod.ModelRunner._capture
+
+    def counted(self, shape, width):
+        captures.append((shape, width))
+        return real(self, shape, width)
+
+    monkeypatch.setattr(runner_mod.ModelRunner, "_capture", counted)
+    steps, where, peak = traces.mixed(seqs, seed=11)
+    thin = [dict(st, entries=[dict(e, want=e["want"][-1:]) for e in st["entries"]]) for st in steps]
+    thin_where = []
+    for st, w in zip(steps, where):
+        at, kept = 0, []
+        for e in st["entries"]:
+            kept += w[at + len(e["want"]) - 1 : at + len(e["want"])]
+            at += len(e["want"])
+        thin_where.append(kept)
+    rep = replay(model, thin, thin_where, ref, torch.bfloat16, peak, page, graphs=True)
+    assert len(rep.runner._graphs) <= 3
+    shapes = [s for s, _ in captures]
+    assert len(set(shapes)) > 3 and len(shapes) > len(set(shapes)), "shapes were meant to be dropped and captured again"
+    widths = [w for _, w in captures]
+    assert max(widths) >= 4 * min(widths) and min(widths) < 16, "block tables were meant to start narrow and grow"
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_graph_and_eager_decode_agree(tiny_folders, name):
     folder, page = tiny_folders[name], TINY[name]["page"]
