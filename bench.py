@@ -250,8 +250,8 @@ def main() -> int:
             points_frac[f"decode_b{b}"] = round(nbytes / (d / k) / 1e9 / HBM_GBPS, 4)
 
     if not a.no_points and a.shape == "8b" and not a.layers:
-        # BASELINE's fourth configuration beside the headline: 32 requests through the Llama-3.2-1B shape, continuous batching
-        # with prompts in portions of 512
+        # the serving workload beside the headline: 32 requests through the Llama-3.2-1B shape, continuous batching with
+        # prompts in portions of 512
         del model
         torch.cuda.empty_cache()
         small = dict(SHAPES["1b"])

@@ -1,6 +1,6 @@
 """One step's batch as the parts see it: flat token arrays, per-request arrays, block tables per cache
-group and the tile lists of the attention kernels, all views of ONE int32 buffer that is filled on the
-host and copied to the device in one piece.
+group and the batch's requests as lists of tiles (for mixers that work tile by tile, as the attention
+kernels do), all views of ONE int32 buffer that is filled on the host and copied to the device in one piece.
 
 Layout of the batch (reference: kv/cache.py:42-61,125-157 builds the same facts as qo_indptr /
 kv_indptr / kv_indices / kv_last_page_len / positions / slots):

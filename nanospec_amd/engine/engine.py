@@ -26,7 +26,7 @@ class EngineConfig:
     block_size: int = 16  # tokens per page
     max_admit: int = 32  # admissions per step
     max_running: int | None = None  # concurrent requests; None = whatever the pool holds (at most 256)
-    cuda_graphs: bool = True  # decode steps replay a captured HIP graph (the reference's name for the option)
+    cuda_graphs: bool = True  # steps replay captured HIP graphs where they can (the reference's name for the option)
     record_logits: bool = False  # keep each request's per-step next-token logits on the CPU (tests)
     profile: bool = False  # per-phase event timings in Engine.prof
     head_chunk: int = 256  # rows per head + sampling pass
