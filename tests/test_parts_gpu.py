@@ -449,6 +449,9 @@ class ParallelBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def max_positions(self):
+        return self.mixer.max_positions()
+
     def forward(self, ctx, resid, delta, cache, owns_cache, delta_out):
         h = self.norm.forward(ctx, resid=resid, x=delta, write_resid=delta is not None)
         a = self.mixer.forward(ctx, h, cache, owns_cache)
@@ -624,3 +627,97 @@ def test_windowed_layers_give_pages_back_while_requests_run(dtype):
     for r in seqs:
         runner.release(r)
     manager.check()
+
+
+# ------------------------------------------------------- a whole architecture that the framework has never heard of
+
+
+@dataclass(frozen=True)
+class ToyParallelConfig:
+    """The configuration of an architecture defined here: blocks with one norm and mixer and feed-forward side by side,
+    config.json keys and tensor names of its own."""
+
+    vocab: int
+    width: int
+    depth: int
+    n_head: int
+    n_kv: int
+    d_head: int
+    d_ff: int
+    eps: float
+    n_ctx: int
+
+    @classmethod
+    def from_hf(cls, cfg, generation_cfg=None):
+        return cls(cfg["vocab"], cfg["width"], cfg["depth"], cfg["n_head"], cfg["n_kv"], cfg["d_head"], cfg["d_ff"], cfg["eps"], cfg["n_ctx"])
+
+    def to_hf(self):
+        return dict(architectures=["ToyParallelLM"], model_type="toy_parallel", **self.__dict__)
+
+    def model_spec(self):
+        import math
+
+        from nanospec_amd.config.spec import AttentionSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
+
+        norm = RMSNormSpec(self.width, self.eps)
+        attn = AttentionSpec(self.width, self.n_head, self.n_kv, self.d_head, RopeSpec(self.d_head, 1e4, max_positions=self.n_ctx),
+                             1 / math.sqrt(self.d_head))
+        layers = tuple(ParallelBlockSpec(f"h.{i}.", norm, attn, SwiGLUSpec(self.width, self.d_ff)) for i in range(self.depth))
+        return ModelSpec(self.vocab, self.width, "wte", layers, tuple(LayerCall(i) for i in range(self.depth)), norm, "ln_f", "out_head", False)
+
+
+def test_an_architecture_registered_from_outside_generates(tmp_path):
+    """A typed configuration, a block class and one registry entry, all defined in this file: the framework writes a model
+    folder with random weights for it, finds the architecture by config.json, loads it by tensor name, generates through
+    the engine and the one-call entry point, and replays a trace; the tokens are the plain functions' greedy choice."""
+    import json
+
+    from nanospec_amd import SamplingParams, generate, load_model
+    from nanospec_amd.config import load_config, register_architecture
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.parts import register
+    from nanospec_amd.weights import write_model_folder
+
+    register("block", "parallel", ParallelBlock)
+    register_architecture("ToyParallelLM", lambda cfg, gen=None: (lambda c: (c, c.model_spec()))(ToyParallelConfig.from_hf(cfg, gen)),
+                          model_type="toy_parallel")
+    config = ToyParallelConfig(vocab=131, width=64, depth=2, n_head=4, n_kv=2, d_head=16, d_ff=96, eps=1e-5, n_ctx=96)
+    folder = write_model_folder(tmp_path / "toy", config, seed=9)
+    assert json.loads((folder / "config.json").read_text())["architectures"] == ["ToyParallelLM"]
+    loaded_cfg, spec = load_config(folder)
+    assert loaded_cfg == config and spec.embed_name == "wte"
+    w = pl.read_safetensors(folder / "model.safetensors")
+    assert "h.1.att.k_proj.weight" in w and "h.0.ln.w" in w
+
+    def plain(tokens):
+        t = len(tokens)
+        x = w["wte"][torch.tensor(tokens)]
+        cos, sin = pl.rotation_tables(torch.arange(t), pl.inverse_frequencies(16, 1e4, None))
+        for i in range(2):
+            p = f"h.{i}."
+            h = pl.rms_norm(x, w[p + "ln.w"], 1e-5)
+            q = pl.rotate(pl.linear(h, w[p + "att.q_proj.weight"]).view(t, 4, 16), cos, sin)
+            k = pl.rotate(pl.linear(h, w[p + "att.k_proj.weight"]).view(t, 2, 16), cos, sin)
+            v = pl.linear(h, w[p + "att.v_proj.weight"]).view(t, 2, 16)
+            a = pl.linear(pl.causal_attention(q, k, v).reshape(t, -1), w[p + "att.o_proj.weight"])
+            f = pl.swiglu(h, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+            x = x + (a + f)
+        return pl.rms_norm(x, w["ln_f"], 1e-5) @ w["out_head"].T
+
+    def plain_greedy(prompt, n):
+        seq = list(prompt)
+        for _ in range(n):
+            seq.append(int(plain(seq)[-1].argmax()))
+        return seq[len(prompt):]
+
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(0, 131, (n,), generator=g).tolist() for n in (4, 19, 33)]
+    want = [plain_greedy(p, 6) for p in prompts]
+    assert generate(str(folder), prompts, SamplingParams(max_tokens=6), dtype="float32", block_size=4, max_step_tokens=24, prefill_chunk=16) == want
+    model = load_model(folder, dtype="float32")
+    assert model.max_positions == 96
+    rep = Replayer(model, 128, page_size=4)
+    out = rep.step([{"id": "a", "tokens": prompts[2][:20], "want": [19]}, {"id": "b", "tokens": prompts[1][:2], "want": []}], [])
+    torch.testing.assert_close(out[0], plain(prompts[2][:20])[-1], rtol=1e-4, atol=1e-4)
+    out = rep.step([{"id": "a", "tokens": prompts[2][20:], "want": [12]}, {"id": "b", "tokens": prompts[1][2:], "want": [16]}], ["a", "b"])
+    torch.testing.assert_close(out, torch.stack([plain(prompts[2])[-1], plain(prompts[1])[-1]]), rtol=1e-4, atol=1e-4)
