@@ -68,8 +68,9 @@ def launch_plans(ctx, group: int, kv_heads: int, head_dim: int) -> list[LaunchPl
         # and where no request can be that long they are not launched: they would cost a captured step 1%)
         items = ctx.n_decode_tiles * kv_heads * -(-group // hp)
         splits = max(1, min(32 if ctx.max_kv_len >= LONG_ROW_KEYS else 16, DECODE_WAVES_PER_UNIT * units // (4 * items)))
-        if not ctx.captured:
-            splits = max(1, min(splits, -(-ctx.max_kv_len // 256)))
+        # never ranges of fewer than 256 keys (in a captured step: of what its block tables can hold): short rows are
+        # short chains already, and a single range needs no kernel to join it
+        splits = max(1, min(splits, -(-ctx.max_kv_len // 256)))
         ws = None
         if splits > 1:
             cols = ctx.n_decode_tiles * (16 // hp) * kv_heads * group
