@@ -125,8 +125,8 @@ def prefill_run(model, cfg, n_tokens: int, block_size: int, reps: int = 3, porti
 
 def serve_run(model, cfg, n_requests: int, new_tokens: int, chunk: int, block_size: int, seed: int = 0, reps: int = 2):
     """Continuous batching with chunked prefill: ``n_requests`` arrive at once with prompts of 16 to 1,024 uniform-random
-    token ids and generate ``new_tokens`` each; prompts are taken in portions of at most ``chunk`` tokens beside the decoding
-    of the requests that are through theirs.  -> (seconds of the best pass, steps, prompt lengths, new tokens)."""
+    token ids and generate ``new_tokens`` each; a step holds at most ``chunk`` tokens: one for every request that is
+    through its prompt, the rest portions of prompts.  -> (seconds of the best pass, steps, prompt lengths, new tokens)."""
     import torch
 
     from nanospec_amd import Engine, EngineConfig, SamplingParams
@@ -139,7 +139,7 @@ def serve_run(model, cfg, n_requests: int, new_tokens: int, chunk: int, block_si
     # One engine for all passes, as a server is one engine for all its requests: the first pass captures the steps' graphs
     # (the reference captures its graphs before it serves), the later ones are timed.
     eng = Engine(model, EngineConfig(num_blocks=n_requests * per_request + 2, block_size=block_size, max_admit=n_requests,
-                                     max_running=n_requests, max_step_tokens=chunk + n_requests, prefill_chunk=chunk,
+                                     max_running=n_requests, max_step_tokens=chunk, prefill_chunk=chunk,
                                      max_seq_len=1024 + new_tokens + block_size))
     for i in range(reps + 1):
         reqs = [eng.add(p, SamplingParams(max_tokens=new_tokens)) for p in prompts]

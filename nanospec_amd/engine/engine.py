@@ -59,6 +59,7 @@ class Engine:
                                config.on_exhaustion)
         self.sched.on_admit = self.runner.admit
         self.sched.on_release = self.runner.release
+        self.sched.decode_rows_cost = self.runner.rows_cost
         self.usable_blocks = config.num_blocks
         if self.runner.use_graphs:
             self.runner._ensure_pad()  # one page is held for pad rows for good (reference: engine/engine.py:101-102)

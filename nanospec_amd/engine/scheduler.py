@@ -10,8 +10,10 @@ A request's tokens are ``prompt + output``; ``computed`` of them are in the cach
 request brings its next tokens: exactly one when it is decoding, a portion when (part of) its prompt is
 still to be computed.  It samples in the step that consumes its last known token.
 
-Token budget (``max_step_tokens``): decoding requests come first with one token each; what is left is
-given to unfinished prompts in admission order, at most ``prefill_chunk`` tokens per request and step.
+Token budget (``max_step_tokens``): decoding requests come first with one token each (counted as
+``decode_rows_cost`` says: the engine rounds them up to the rows of a captured step, so that a step with its
+padding stays within the budget); what is left is given to unfinished prompts in admission order, at most
+``prefill_chunk`` tokens per request and step.
 When the budget does not even cover the decoding requests, those that have waited longest since their
 last step go first (so that all of them advance in turn), and an eighth of the budget (at least one
 token) is kept for the oldest unfinished prompt, so that it advances too.
@@ -104,6 +106,9 @@ class Scheduler:
         # hooks the engine sets so that device state follows admission and release
         self.on_admit = cache.admit
         self.on_release = cache.release
+        # what so many rows of one token take of a step's token budget: the engine pads them to the size of a captured
+        # step, and a step padded beyond the budget would cost more than the budget was meant to allow
+        self.decode_rows_cost = lambda n: n
 
     @property
     def has_work(self) -> bool:
@@ -185,16 +190,18 @@ class Scheduler:
         work: list[Work] = []
         decoding = [r for r in self.running if r.seq_len - r.computed == 1]
         filling = [r for r in self.running if r.seq_len - r.computed > 1]
-        if budget is not None and len(decoding) + (1 if filling else 0) > budget:
+        cost = self.decode_rows_cost
+        if budget is not None and cost(len(decoding)) + (1 if filling else 0) > budget:
             # not every decoding request fits: the longest-waiting first, and a share for the oldest unfinished prompt
             share = max(1, budget // 8) if filling and budget > 1 else 0
-            decoding = sorted(decoding, key=lambda r: r.served_at)[: budget - share]
+            fit = len(decoding)
+            while fit and cost(fit) > budget - share:
+                fit -= 1
+            decoding = sorted(decoding, key=lambda r: r.served_at)[:fit]
         for r in decoding:
-            if budget is not None and budget <= 0:
-                break
             work.append(Work(r, r.computed, 1))
-            if budget is not None:
-                budget -= 1
+        if budget is not None:
+            budget -= cost(len(decoding))
         for r in filling:
             n = r.seq_len - r.computed
             if self.prefill_chunk is not None:

@@ -148,6 +148,35 @@ def test_a_prompt_advances_although_the_decoding_requests_fill_the_budget():
     assert ids(run_step(s2))[-1] == (8, 12)
 
 
+def test_decoding_rows_count_as_the_engine_pads_them():
+    """The engine rounds the rows of decoding requests up to a captured step's size and says so through ``decode_rows_cost``:
+    the budget is then charged for the padded rows, so a step with its padding stays within it, and when not all decoding
+    requests fit it takes as many as fit with their padding."""
+    buckets = (1, 2, 4, 8)
+    cost = lambda n: next((b for b in buckets if b >= n), n) if n else 0
+    s = Scheduler(manager(256, 4), max_admit=16, max_step_tokens=32)
+    s.decode_rows_cost = cost
+    for i in range(5):
+        s.add(req(i, 1, max_tokens=40))
+    run_step(s)
+    s.add(req(5, 100, max_tokens=2))
+    work = run_step(s)
+    assert ids(work) == [(i, 1) for i in range(5)] + [(5, 24)]  # five rows are padded to eight: 24 of 32 are left
+    # a budget of six: five rows would be padded to eight, so four go (padded to four) and the prompt has the rest
+    s = Scheduler(manager(256, 4), max_admit=16, max_step_tokens=6)
+    s.decode_rows_cost = cost
+    for i in range(5):
+        s.add(req(i, 1, max_tokens=40))
+    run_step(s), run_step(s)  # prompts of one token: two steps under this budget
+    s.add(req(5, 100, max_tokens=2))
+    for _ in range(6):
+        work = run_step(s)
+        n_dec = sum(1 for w in work if w.req.id != 5)
+        assert cost(n_dec) + sum(w.n for w in work if w.req.id == 5) <= 6
+        assert any(w.req.id == 5 for w in work)
+    assert max(len(r.out_tokens) for r in s.running if r.id != 5) - min(len(r.out_tokens) for r in s.running if r.id != 5) <= 1
+
+
 def test_preemption_when_pages_run_out():
     """Under "preempt" admission needs only the first portion.  When a step does not fit, the request admitted last goes
     back to the HEAD of the queue with its output kept; later it is recomputed from prompt + output."""
