@@ -547,6 +547,41 @@ extern "C" int ns_silu_mul(void* out, const void* gu, int n_rows, int inter, int
   return ns_launch_status();
 }
 
+// A weight matrix back from the layout of the streaming kernels (gemm_bf16.hip:
+// wt[rt][kt][i][lane = 16 g + r][e] = w[16 rt + r][128 kt + 32 g + 8 i + e]) into plain rows [N, K], for a library product
+// over many rows where only the re-laid copy is kept.  One wave per tile of 16 rows x 128 k: four loads of a contiguous
+// kilobyte each; a lane then holds 32 consecutive elements of one row and writes them as 64 contiguous bytes, the four
+// lanes of a row 256.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 untile_piece;
+__global__ __launch_bounds__(256) void untile_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ wt, int N, int K,
+                                                     int KT, long tiles) {
+  const int lane = threadIdx.x & 63;
+  const long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= tiles) return;
+  const int rt = (int)(tile / KT), kt = (int)(tile % KT);
+  const int r = lane & 15, g = lane >> 4;
+  const bf16_t* src = wt + (size_t)tile * (16 * 128) + (size_t)lane * 8;
+  untile_piece v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const untile_piece*>(src + i * 64 * 8);
+  const int row = rt * 16 + r;
+  if (row >= N) return;
+  bf16_t* dst = out + (size_t)row * K + kt * 128 + g * 32;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (kt * 128 + g * 32 + i * 8 < K) *reinterpret_cast<untile_piece*>(dst + i * 8) = v[i];  // K is a multiple of 8
+}
+// out: [N, K] bfloat16, contiguous, 16-byte aligned; wt: the re-laid matrix (rows padded to 16, k to 128).
+extern "C" int ns_untile_bf16(void* out, const void* wt, int N, int K, hipStream_t stream) {
+  if (N <= 0 || K <= 0 || (K & 7) || (((uintptr_t)out | (uintptr_t)wt) & 15)) return NS_ERR_BAD_ARG;
+  const int KT = (K + 127) / 128;
+  const long tiles = (long)((N + 15) / 16) * KT;
+  const long blocks = (tiles + 3) / 4;
+  if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
+  untile_kernel<<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)wt, N, K, KT, tiles);
+  return ns_launch_status();
+}
+
 // A fill kernel for 32-bit words: graphs must not hold memset nodes, so buffers that a captured step
 // clears are cleared with this.
 __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n) {

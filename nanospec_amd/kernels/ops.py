@@ -278,6 +278,16 @@ class TiledWeight:
         return out
 
 
+def untile(w: TiledWeight, out: torch.Tensor) -> torch.Tensor:
+    """The matrix of ``w`` in plain rows, into ``out`` [n, k] (bfloat16, contiguous): what a library product over many rows
+    reads, made for the one product where only the re-laid copy is kept."""
+    _gpu(out)
+    if out.dtype != torch.bfloat16 or out.shape != (w.n, w.k) or not out.is_contiguous() or out.data_ptr() % 16 or w.k % 8:
+        raise KernelRefused(f"untile: out must be a contiguous bfloat16 [{w.n}, {w.k}], 16-byte aligned, k a multiple of 8")
+    _check(build.core().ns_untile_bf16(_ptr(out), _ptr(w.data), c_int(w.n), c_int(w.k), _stream()), "untile")
+    return out
+
+
 def tiled_takes(x: torch.Tensor, k: int, max_rows: int = SKINNY_MAX_ROWS) -> bool:
     return (x.dtype == torch.bfloat16 and x.shape[0] <= max_rows and k % 8 == 0 and x.stride(0) % 8 == 0
             and x.stride(1) == 1 and x.data_ptr() % 16 == 0)

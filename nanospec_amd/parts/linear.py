@@ -30,6 +30,11 @@ STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the sha
 WIDE_HEAD_ROWS = 12  # above this many rows a wide 32-bit product (the head) is faster through the 17-to-64-row kernel
 WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
 #                    32-bit results, which the library does not give); wider products go to the library
+UNTILE_MIN_ROWS = 768  # where only the re-laid copy is kept: from this many rows on the products whose callers allow it
+#                        (``plain_copy``: q/k/v, o, gate/up) first write their matrices out in plain rows (scratch) and go to
+#                        the library; the copy costs what 300 rows of the product cost, and the library is 1.6 to 2 times as
+#                        fast as the many-row kernel (measured for these at the 70B shape; the down-projection's comparison
+#                        is missing, so it stays with the many-row kernel)
 
 
 class IntoResidual:
@@ -68,8 +73,9 @@ class LinearWeight:
         """Whether a product of ``rows`` rows can take a ``PreNormed`` input and can end in the residual stream."""
         return self.tiled is not None and rows <= STREAM_ROWS
 
-    def into_residual(self, x: torch.Tensor, link: IntoResidual, arena=None):
-        """x @ W^T on its way into the residual stream, in one of the forms ``IntoResidual`` names."""
+    def into_residual(self, x: torch.Tensor, link: IntoResidual, arena=None, plain_copy: bool = False):
+        """x @ W^T on its way into the residual stream, in one of the forms ``IntoResidual`` names.  ``plain_copy``: as for
+        ``__call__``."""
         m = x.shape[0]
         take = (lambda shape, dtype: arena.take(shape, dtype)) if arena is not None else (lambda shape, dtype: torch.empty(shape, dtype=dtype, device=x.device))
         if self.links_norms(m) and x.dtype == torch.bfloat16 and ops.tiled_takes(x[:1], self.k):
@@ -88,18 +94,23 @@ class LinearWeight:
             if ws is not None:
                 return ops.linear_wide(x, self.tiled, workspace=ws, ksplit=ksplit, nt=nt, defer=True)
         r = link.resid
-        if (m > ops.SKINNY_MAX_ROWS and self._plain_t is not None and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16
+        plain_t = self._plain_t
+        if (plain_t is None and plain_copy and self.tiled is not None and m >= UNTILE_MIN_ROWS and x.dtype == torch.bfloat16
+                and ops.tiled_takes(x[:1], self.k)):
+            plain_t = ops.untile(self.tiled, take((self.n, self.k), self.dtype)).t()  # only the re-laid copy is kept, many rows
+        if (m > ops.SKINNY_MAX_ROWS and plain_t is not None and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16
                 and r.shape == (m, self.n) and r.is_contiguous()):
             # many rows: the library's product takes the stream as its addend, resid = resid + x @ W^T summed in 32-bit and
             # rounded once, so the norm after it reads one tensor instead of two and writes one instead of two
-            r.addmm_(x, self._plain_t)
+            r.addmm_(x, plain_t)
             return ops.Added()
         out = link.x_next if link.x_next is not None else take((m, self.n), x.dtype)
         return self(x, out=out, arena=arena)
 
-    def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None) -> torch.Tensor:
+    def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None, plain_copy: bool = False) -> torch.Tensor:
         """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated.
-        ``x`` may be a ``PreNormed`` where ``links_norms`` holds."""
+        ``x`` may be a ``PreNormed`` where ``links_norms`` holds.  ``plain_copy``: where only the re-laid copy is kept, many
+        rows may go to the library through a plain copy of the matrix in scratch (see ``UNTILE_MIN_ROWS``)."""
         if isinstance(x, ops.PreNormed):
             if not self.links_norms(x.shape[0]):
                 raise ops.KernelRefused("this product cannot take a pre-normed input (rows, layout or precision)")
@@ -128,7 +139,10 @@ class LinearWeight:
             return torch.matmul(x, self._plain_t) if out is None else torch.matmul(x, self._plain_t, out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
-        if m > ops.WIDE_TALL_ROWS:  # only the tiled layout is kept: blocks of 128 rows through the hand-written kernel
+        if m >= UNTILE_MIN_ROWS and not out_f32 and plain_copy:  # only the tiled layout is kept, many rows: a plain copy for this one product
+            plain = arena.take((self.n, self.k), self.dtype) if arena is not None else torch.empty((self.n, self.k), dtype=self.dtype, device=x.device)
+            return torch.matmul(x, ops.untile(self.tiled, plain).t(), out=out)
+        if m > ops.WIDE_TALL_ROWS:  # ... fewer: blocks of 128 rows through the hand-written kernel
             ksplit, nt = ops.rows_plan(self.n, self.k, m)
             ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
             return ops.linear_rows(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
@@ -166,6 +180,14 @@ class GatedWeights:
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
+        if fast and self.stacked is None and m >= UNTILE_MIN_ROWS:
+            # only the tiled layout is kept, many rows: both matrices in plain rows into scratch, then as with both layouts
+            stacked = ctx.arena.take((2 * self.inter, self.k), x.dtype)
+            ops.untile(self.tiled[0], stacked[: self.inter])
+            ops.untile(self.tiled[1], stacked[self.inter :])
+            gu = ctx.arena.take((m, 2 * self.inter), x.dtype)
+            torch.matmul(x, stacked.t(), out=gu)
+            return ops.silu_mul(gu, out=out)
         if fast and self.stacked is None and m > ops.WIDE_TALL_ROWS:
             # only the tiled layout is kept: blocks of 128 rows through the hand-written kernel, activation in the same pass
             return ops.linear_rows(x, self.tiled[0], w2=self.tiled[1], out=out, ksplit=1, nt=2)

@@ -67,7 +67,7 @@ class DecoderModel:
             layouts = "both" if 2.2 * linear + size * 2 * spec.vocab_size * spec.hidden < 0.8 * free else "tiled"
             if layouts == "tiled" and dtype == torch.bfloat16:
                 print(f"[nanospec_amd] {linear / 2**30:.0f} GiB of matrices, {free / 2**30:.0f} GiB free: keeping one layout; "
-                      "steps of many tokens will be slower", file=sys.stderr, flush=True)
+                      "steps of many tokens copy matrices into plain rows first and are slower", file=sys.stderr, flush=True)
         self.layouts = layouts
         get = source.get
         self.embed = get(spec.embed_name).to(device=device, dtype=dtype).contiguous()

@@ -537,6 +537,21 @@ def test_attention_generic(dtype, case, heads, kvh, hd, page):
         assert ulps_of_row_max(out.cpu(), ref).max() <= 4  # the reference's bound, tests/test_backends.py:71
 
 
+@pytest.mark.parametrize("n,k", [(16, 128), (40, 72), (100, 264), (2048, 8192), (33, 8)])
+def test_untile_gives_the_matrix_back(n, k):
+    """The re-laid copy of a matrix written out in plain rows again (rows and k that are no multiples of the tile: the
+    padding is not written, and nothing outside the matrix is)."""
+    ops = _ops()
+    torch.manual_seed(n + k)
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    guard = torch.full((n + 2, k), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = ops.untile(ops.TiledWeight(w), guard[1:-1])
+    assert torch.equal(out, w)
+    assert bool((guard[0] == 7).all()) and bool((guard[-1] == 7).all())
+    with pytest.raises(ops.KernelRefused):
+        ops.untile(ops.TiledWeight(w), torch.empty(n, k + 8, dtype=torch.bfloat16, device=DEV))
+
+
 def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0,
               chunk_splits=1):
     n = sum(lens)

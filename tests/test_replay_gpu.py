@@ -478,6 +478,43 @@ def test_real_shape_slice_matches_plain(llama_1b_slice, dtype, request):
         assert seen == {"unadded": 0, "linked": 0}
 
 
+def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch):
+    """A model that keeps the re-laid matrices only, a prompt of 800 tokens in one step: q/k/v and gate/up are written out
+    in plain rows for the library's product, o likewise (the library adds into the residual stream), the down-projection
+    runs in blocks through the many-row kernel; then a portion of 200 tokens (blocks only) and single tokens."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.kernels import ops
+    from nanospec_amd.loader import load_model
+
+    folder, dtype = llama_1b_slice, torch.bfloat16
+    cfg, w = pl.read_config(folder), pl.read_weights(folder, dtype)
+    w = {k: (v if v.dim() == 1 else v.float()) for k, v in w.items()}  # the stored values, converted once
+    toks = random_tokens(1010, 128256, 5)
+    places = [0, 1, 511, 767, 799, 800, 950, 999, 1000, 1003, 1009]
+    ref = pl.logits_of_sequence(w, cfg, toks, dtype)[places]
+    at = {p: ref[i] for i, p in enumerate(places)}
+    model = load_model(folder, dtype=dtype, layouts="tiled")
+    calls = {"untile": 0, "rows": 0}
+    real_untile, real_rows = ops.untile, ops.linear_rows
+    monkeypatch.setattr(ops, "untile", lambda *a, **k: (calls.__setitem__("untile", calls["untile"] + 1), real_untile(*a, **k))[1])
+    monkeypatch.setattr(ops, "linear_rows", lambda *a, **k: (calls.__setitem__("rows", calls["rows"] + 1), real_rows(*a, **k))[1])
+    rep = Replayer(model, 1024, page_size=16)
+
+    def step(s, e):
+        wants = [p - s for p in places if s <= p < e]
+        out = rep.step([{"id": "a", "tokens": toks[s:e], "want": wants}], [])
+        if wants:
+            check(out, torch.stack([at[s + i] for i in wants]), dtype, f"tokens {s}:{e}")
+
+    step(0, 800)
+    assert calls == {"untile": 2 * 4, "rows": 2 * 1}, calls  # per layer: q/k/v, o, gate and up; the down-projection
+    step(800, 1000)
+    assert calls["untile"] == 8 and calls["rows"] > 2, calls
+    for p in range(1000, 1010):
+        step(p, p + 1)
+    rep.manager.check()
+
+
 @pytest.fixture(scope="module")
 def llama_8b_slice(tmp_path_factory):
     """Two layers of the Llama-3.1-8B shape (width 4096, 32 heads over 8 key/value heads of 128, feed-forward 14336,
