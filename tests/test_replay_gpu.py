@@ -530,6 +530,41 @@ def llama_8b_slice(tmp_path_factory):
     return write_model_folder(tmp_path_factory.mktemp("llama8b") / "m", LlamaConfig.from_hf(cfg), seed=4, dtype=torch.bfloat16)
 
 
+def test_a_captured_step_of_512_rows_replayed_over_and_over(llama_8b_slice):
+    """The benchmark's layer sizes in the step that serving repeats most often: 32 decode rows beside a prompt portion of 480
+    tokens, 512 rows through the library's products inside a captured graph.  The same captured step is replayed six
+    times with new tokens, longer contexts and other work on the GPU in between, and every replay is compared with the
+    same step launched kernel by kernel in a second cache (a captured library call that keeps state between replays,
+    or a node that is not replayed, would show from the second replay on)."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.loader import load_model
+
+    model = load_model(llama_8b_slice, dtype=torch.bfloat16)
+    vocab = pl.read_config(llama_8b_slice)["vocab"]
+    graphs = Replayer(model, 8192, page_size=16, use_graphs=True, max_live=40)
+    eager = Replayer(model, 8192, page_size=16, use_graphs=False, max_live=40)
+    rows = {f"d{i}": random_tokens(8 + 7, vocab, 900 + i) for i in range(32)}
+    prompt = random_tokens(6 * 480, vocab, 77)
+
+    def both(entries):
+        a, b = graphs.step(entries, []), eager.step(entries, [])
+        torch.cuda.synchronize()
+        return a, b
+
+    both([{"id": r, "tokens": t[:8], "want": []} for r, t in rows.items()])
+    for k in range(6):
+        entries = [{"id": r, "tokens": t[8 + k : 9 + k], "want": [0]} for r, t in rows.items()]
+        entries.append({"id": "p", "tokens": prompt[480 * k : 480 * (k + 1)], "want": [0, 479]})
+        a, b = both(entries)
+        assert graphs.runner.last_used_graph and not eager.runner.last_used_graph
+        check(a, b, torch.bfloat16, f"replay {k}")
+        # other work on the GPU between the replays, of the program's own kind: a decode-only step of the same requests'
+        # cache would change it, so a product of the library on unrelated data
+        junk = torch.randn(300, 4096, dtype=torch.bfloat16, device="cuda")
+        (junk @ junk.t()).sum().item()
+    assert (32, 480) in graphs.runner._graphs  # one captured step served all six
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_benchmark_shape_slice_matches_plain(llama_8b_slice, dtype):
     """The layer sizes of the benchmark end to end: a portion of 280 tokens, a mixed step, decoding with 8 live requests
