@@ -165,7 +165,7 @@ class Attention:
             ops.rope_kv_from_partial(part, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
                                      s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         else:
-            self.wqkv(x, out=qkv, arena=ctx.arena, plain_copy=True)
+            self.wqkv(x, out=qkv, arena=ctx.arena, plain_copy=not ctx.captured)
             ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
                               s.head_dim, pos.rotary_dim, write_kv=owns_cache)
         att = ctx.arena.take((n, s.heads * s.head_dim), x.dtype)
@@ -180,8 +180,8 @@ class Attention:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)
         if residual is not None:
-            return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=True)
-        return self.wo(att, out=out, arena=ctx.arena, plain_copy=True)
+            return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=not ctx.captured)
+        return self.wo(att, out=out, arena=ctx.arena, plain_copy=not ctx.captured)
 
 
 registry.register("mixer", "attention", Attention)

@@ -34,7 +34,8 @@ UNTILE_MIN_ROWS = 768  # where only the re-laid copy is kept: from this many row
 #                        (``plain_copy``: q/k/v, o, gate/up) first write their matrices out in plain rows (scratch) and go to
 #                        the library; the copy costs what 300 rows of the product cost, and the library is 1.6 to 2 times as
 #                        fast as the many-row kernel (measured for these at the 70B shape; the down-projection's comparison
-#                        is missing, so it stays with the many-row kernel)
+#                        is missing, so it stays with the many-row kernel).  Callers allow it in steps that are launched kernel
+#                        by kernel only: the scratch is as large as the matrix, and every captured step keeps its own.
 
 
 class IntoResidual:
@@ -180,8 +181,9 @@ class GatedWeights:
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
-        if fast and self.stacked is None and m >= UNTILE_MIN_ROWS:
+        if fast and self.stacked is None and m >= UNTILE_MIN_ROWS and not ctx.captured:
             # only the tiled layout is kept, many rows: both matrices in plain rows into scratch, then as with both layouts
+            # (not in a captured step: every captured shape would hold a scratch of its own as large as the two matrices)
             stacked = ctx.arena.take((2 * self.inter, self.k), x.dtype)
             ops.untile(self.tiled[0], stacked[: self.inter])
             ops.untile(self.tiled[1], stacked[self.inter :])

@@ -479,9 +479,10 @@ def test_real_shape_slice_matches_plain(llama_1b_slice, dtype, request):
 
 
 def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch):
-    """A model that keeps the re-laid matrices only, a prompt of 800 tokens in one step: q/k/v and gate/up are written out
-    in plain rows for the library's product, o likewise (the library adds into the residual stream), the down-projection
-    runs in blocks through the many-row kernel; then a portion of 200 tokens (blocks only) and single tokens."""
+    """A model that keeps the re-laid matrices only.  A prompt portion of 1,100 tokens, launched kernel by kernel: q/k/v, o
+    and gate/up are written out in plain rows for the library's product (o's adds into the residual stream), the
+    down-projection runs in blocks through the many-row kernel.  A portion of 800 tokens, a captured step: no plain copies,
+    every product in blocks.  Then 100 tokens and single ones."""
     from nanospec_amd.engine.replay import Replayer
     from nanospec_amd.kernels import ops
     from nanospec_amd.loader import load_model
@@ -489,16 +490,20 @@ def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch):
     folder, dtype = llama_1b_slice, torch.bfloat16
     cfg, w = pl.read_config(folder), pl.read_weights(folder, dtype)
     w = {k: (v if v.dim() == 1 else v.float()) for k, v in w.items()}  # the stored values, converted once
-    toks = random_tokens(1010, 128256, 5)
-    places = [0, 1, 511, 767, 799, 800, 950, 999, 1000, 1003, 1009]
-    ref = pl.logits_of_sequence(w, cfg, toks, dtype)[places]
+    toks = random_tokens(2010, 128256, 5)
+    places = [0, 1, 511, 767, 1099, 1100, 1500, 1899, 1900, 1999, 2000, 2003, 2009]
+    x = w["model.embed_tokens.weight"][torch.tensor(toks)].to(dtype)
+    cos, sin = pl.rotation_tables(torch.arange(len(toks)), pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"]))
+    for i in range(cfg["layers"]):
+        x = pl.decoder_layer(x, w, f"model.layers.{i}.", cfg, cos, sin)
+    ref = pl.rms_norm(x[places], w["model.norm.weight"], cfg["eps"]).float() @ w["lm_head.weight"].T
     at = {p: ref[i] for i, p in enumerate(places)}
     model = load_model(folder, dtype=dtype, layouts="tiled")
     calls = {"untile": 0, "rows": 0}
     real_untile, real_rows = ops.untile, ops.linear_rows
     monkeypatch.setattr(ops, "untile", lambda *a, **k: (calls.__setitem__("untile", calls["untile"] + 1), real_untile(*a, **k))[1])
     monkeypatch.setattr(ops, "linear_rows", lambda *a, **k: (calls.__setitem__("rows", calls["rows"] + 1), real_rows(*a, **k))[1])
-    rep = Replayer(model, 1024, page_size=16)
+    rep = Replayer(model, 2048, page_size=16)
 
     def step(s, e):
         wants = [p - s for p in places if s <= p < e]
@@ -506,11 +511,15 @@ def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch):
         if wants:
             check(out, torch.stack([at[s + i] for i in wants]), dtype, f"tokens {s}:{e}")
 
-    step(0, 800)
+    step(0, 1100)
+    assert not rep.runner.last_used_graph
     assert calls == {"untile": 2 * 4, "rows": 2 * 1}, calls  # per layer: q/k/v, o, gate and up; the down-projection
-    step(800, 1000)
-    assert calls["untile"] == 8 and calls["rows"] > 2, calls
-    for p in range(1000, 1010):
+    step(1100, 1900)
+    assert rep.runner.last_used_graph
+    # (the step ran three times: twice before its capture and once from the graph, whose kernels do not pass through here)
+    assert calls["untile"] == 8 and calls["rows"] > 2 and calls["rows"] % 4 == 2, calls  # q/k/v, o, gate/up, down: all in blocks
+    step(1900, 2000)
+    for p in range(2000, 2010):
         step(p, p + 1)
     rep.manager.check()
 
