@@ -574,6 +574,33 @@ def test_a_captured_step_of_512_rows_replayed_over_and_over(llama_8b_slice):
     assert (32, 480) in graphs.runner._graphs  # one captured step served all six
 
 
+def test_a_captured_decode_step_of_208_rows_replayed_over_and_over(llama_8b_slice):
+    """The benchmark's layer sizes with 200 live requests: decode steps of more than 128 rows run their products through the
+    library inside a captured graph (few rows, inner sizes of 4,096 and 14,336: shapes for which a library may cut the
+    inner size and keep partial results in a workspace of its own).  Five replays with new tokens, each compared with the
+    same step launched kernel by kernel in a second cache."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.loader import load_model
+
+    model = load_model(llama_8b_slice, dtype=torch.bfloat16)
+    vocab = pl.read_config(llama_8b_slice)["vocab"]
+    graphs = Replayer(model, 200 * 64, page_size=16, use_graphs=True, max_live=200)
+    eager = Replayer(model, 200 * 64, page_size=16, use_graphs=False, max_live=200)
+    rows = {f"d{i}": random_tokens(3 + i % 5 + 5, vocab, 300 + i) for i in range(200)}
+    for at in range(0, 200, 50):  # prompts, fifty requests a step
+        entries = [{"id": r, "tokens": t[:-5], "want": []} for r, t in list(rows.items())[at : at + 50]]
+        graphs.step(entries, []), eager.step(entries, [])
+    for k in range(5):
+        entries = [{"id": r, "tokens": [t[len(t) - 5 + k]], "want": [0]} for r, t in rows.items()]
+        a, b = graphs.step(entries, []), eager.step(entries, [])
+        torch.cuda.synchronize()
+        assert graphs.runner.last_used_graph and not eager.runner.last_used_graph
+        check(a, b, torch.bfloat16, f"replay {k}")
+        junk = torch.randn(300, 4096, dtype=torch.bfloat16, device="cuda")
+        (junk @ junk.t()).sum().item()
+    assert (208, 0) in graphs.runner._graphs
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_benchmark_shape_slice_matches_plain(llama_8b_slice, dtype):
     """The layer sizes of the benchmark end to end: a portion of 280 tokens, a mixed step, decoding with 8 live requests
