@@ -3,6 +3,7 @@ the output head (reference: model/llama.py:211-286).  Nothing here knows an arch
 
 from __future__ import annotations
 
+import math
 import sys
 
 import torch
@@ -62,7 +63,7 @@ class DecoderModel:
             raise ValueError(f"layouts={layouts!r}: use 'auto', 'both' or 'tiled'")
         if layouts == "auto":
             size = torch.finfo(dtype).bits // 8
-            linear = sum(size * shape[0] * shape[1] for name, (shape, role) in full.items() if role == "linear" and name != spec.head_name)
+            linear = sum(size * math.prod(shape) for name, (shape, role) in full.items() if role == "linear" and name != spec.head_name)
             free = torch.cuda.mem_get_info(self.device)[0]
             layouts = "both" if 2.2 * linear + size * 2 * spec.vocab_size * spec.hidden < 0.8 * free else "tiled"
             if layouts == "tiled" and dtype == torch.bfloat16:

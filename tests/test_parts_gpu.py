@@ -1,7 +1,7 @@
 """Each kind of part alone against the plain function it implements, at sizes of its own; a model put together from
 parts in an unusual order (a layer run twice, an entry that reads another entry's cache); and a toy mixer with state of
-its own, a toy feed-forward with routing and a toy position encoding that are defined here, registered, built and stepped
-without touching the framework."""
+its own, a toy feed-forward with routing, a toy position encoding and a toy norm that are defined here, registered, built
+and stepped without touching the framework."""
 
 from __future__ import annotations
 
@@ -408,6 +408,112 @@ def test_toy_routed_feed_forward_and_toy_position_in_one_layer_only():
         want = torch.cat([refs[r][s:e] for r, s, e in entries])
         err = ((out.cpu() - want).abs().amax(-1) / want.abs().amax(-1)).max()
         assert err < 1e-4, (entries, float(err))
+
+
+# ------------------------------------------------------- a toy norm
+
+
+@dataclass(frozen=True)
+class CentredNormSpec:
+    """y = weight * (r - mean(r)) / sqrt(var(r) + eps) + bias over the channels of a row."""
+
+    kind: ClassVar[str] = "centred"
+    dim: int
+    eps: float
+
+
+class CentredNorm:
+    """Takes what every norm of a pre-norm block takes: the stream, what is still to be added to it, the rows to give.
+    It does not say ``links_products``, so the products around it neither fold its factor in nor hand it unadded ranges."""
+
+    graph_safe = True
+
+    def __init__(self, spec, name):
+        self.spec, self.name, self.bias_name = spec, name, name.replace("weight", "bias")
+
+    def wanted(self):
+        return {self.name: ((self.spec.dim,), "norm"), self.bias_name: ((self.spec.dim,), "linear")}
+
+    def load(self, get, dtype, device):
+        self.weight = get(self.name).to(device=device, dtype=dtype)
+        self.bias = get(self.bias_name).to(device=device, dtype=dtype)
+
+    def forward(self, ctx, resid=None, x=None, rows=None, write_resid=False, out=None):
+        assert x is None or isinstance(x, torch.Tensor), type(x)  # never a product's unadded ranges
+        r = resid if x is None else (resid.float() + x.float()).to(resid.dtype)
+        if write_resid:
+            resid.copy_(r)
+        if rows is not None:
+            r = r[rows.long()]
+        f = r.float()
+        y = (f - f.mean(-1, keepdim=True)) * torch.rsqrt(f.var(-1, unbiased=False, keepdim=True) + self.spec.eps)
+        y = (y * self.weight.float() + self.bias.float()).to(r.dtype)
+        return y if out is None else out.copy_(y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_toy_norm_in_one_layer_and_at_the_end(dtype):
+    """A norm of another kind, registered from here: both norms of the second layer and the norm before the head.  The first
+    layer keeps RMS norms, whose products fold the norm in where they can (few rows, bfloat16) and must stop doing so at
+    the border to the other kind."""
+    import math
+
+    from nanospec_amd.config.spec import AttentionSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.parts import DecoderModel, register
+    from nanospec_amd.weights import DictSource, random_tensors
+
+    register("norm", "centred", CentredNorm)
+    hidden, vocab, hd, inner = 64, 83, 16, 88
+    rms, centred = RMSNormSpec(hidden, 1e-5), CentredNormSpec(hidden, 1e-3)
+    attn = AttentionSpec(hidden, 4, 2, hd, RopeSpec(hd, 1e4), 1 / math.sqrt(hd))
+    layers = (llama_block("model.layers.0.", rms, attn, rms, SwiGLUSpec(hidden, inner)),
+              llama_block("model.layers.1.", centred, attn, centred, SwiGLUSpec(hidden, inner)),
+              llama_block("model.layers.2.", rms, attn, rms, SwiGLUSpec(hidden, inner)))
+    spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers, (LayerCall(0), LayerCall(1), LayerCall(2)), centred,
+                     "model.norm.weight", "lm_head.weight", False)
+    net = DecoderModel(spec)
+    wanted = net.wanted()
+    assert "model.layers.1.input_layernorm.bias" in wanted and "model.norm.bias" in wanted and "model.layers.0.input_layernorm.bias" not in wanted
+    w = random_tensors(wanted, seed=5)
+    w = {k: (v * 6.0 if "proj" in k else v + (0.3 if k.endswith("bias") else 0.0)).to(dtype) for k, v in w.items()}
+    model = net.load(DictSource(w), dtype, DEV)
+
+    def centred_norm(x, name, eps):
+        f = x.float()
+        y = (f - f.mean(-1, keepdim=True)) * torch.rsqrt(f.var(-1, unbiased=False, keepdim=True) + eps)
+        return (y * w[name].float() + w[name.replace("weight", "bias")].float()).to(x.dtype)
+
+    def plain(tokens):
+        t = len(tokens)
+        x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        cos, sin = pl.rotation_tables(torch.arange(t), pl.inverse_frequencies(hd, 1e4, None))
+        for i in range(3):
+            p = f"model.layers.{i}."
+            norm = (lambda y, name: centred_norm(y, name, 1e-3)) if i == 1 else (lambda y, name: pl.rms_norm(y, w[name], 1e-5))
+            h = norm(x, p + "input_layernorm.weight")
+            q = pl.rotate(pl.linear(h, w[p + "self_attn.q_proj.weight"]).view(t, 4, hd), cos, sin)
+            k = pl.rotate(pl.linear(h, w[p + "self_attn.k_proj.weight"]).view(t, 2, hd), cos, sin)
+            v = pl.linear(h, w[p + "self_attn.v_proj.weight"]).view(t, 2, hd)
+            x = x + pl.linear(pl.causal_attention(q, k, v).reshape(t, -1), w[p + "self_attn.o_proj.weight"])
+            h = norm(x, p + "post_attention_layernorm.weight")
+            x = x + pl.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        return centred_norm(x, "model.norm.weight", 1e-3).float() @ w["lm_head.weight"].float().T
+
+    g = torch.Generator().manual_seed(9)
+    seqs = {r: torch.randint(0, vocab, (n,), generator=g).tolist() for r, n in (("a", 60), ("b", 23))}
+    refs = {r: plain(t) for r, t in seqs.items()}
+    rep = Replayer(model, 128, page_size=8)
+    steps = [[("a", 0, 40), ("b", 0, 2)], [("a", 40, 41), ("b", 2, 22)]] + [[("a", 41 + i, 42 + i)] + ([("b", 22, 23)] if i == 0 else []) for i in range(19)]
+    for entries in steps:
+        out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(range(e - s))} for r, s, e in entries], [])
+        want = torch.cat([refs[r][s:e] for r, s, e in entries])
+        if dtype == torch.float32:
+            err = ((out.cpu() - want).abs().amax(-1) / want.abs().amax(-1)).max()
+            assert err < 1e-4, (entries, float(err))
+        else:
+            assert ulps_of_row_max(out.cpu(), want).max() <= 8, entries
+    assert rep.runner.last_used_graph  # the single-token steps were captured with the toy norm inside
 
 
 # ------------------------------------------------------- a toy block of another shape, and tensor names of another origin
