@@ -277,6 +277,61 @@ def test_toy_mixer_with_state_layer_twice_and_borrowed_cache():
     rep.manager.check()
 
 
+def test_a_model_without_any_paged_cache():
+    """Every layer's mixer keeps a state of fixed size and nothing in pages (the shape of a recurrent architecture): no group
+    of pages exists, requests still get slots, steps and the scheduler run as for any model."""
+    from nanospec_amd import Engine, EngineConfig, SamplingParams
+    from nanospec_amd.config.spec import LayerCall, ModelSpec, RMSNormSpec, SwiGLUSpec
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.parts import DecoderModel, register
+    from nanospec_amd.weights import DictSource, random_tensors
+
+    register("mixer", "prefix_mean", PrefixMean)
+    hidden, vocab = 40, 53
+    norm = RMSNormSpec(hidden, 1e-5)
+    layers = tuple(llama_block(f"model.layers.{i}.", norm, PrefixMeanSpec(hidden), norm, SwiGLUSpec(hidden, 56)) for i in range(2))
+    spec = ModelSpec(vocab, hidden, "model.embed_tokens.weight", layers, (LayerCall(0), LayerCall(1)), norm, "model.norm.weight",
+                     "lm_head.weight", False)
+    net = DecoderModel(spec)
+    w = random_tensors(net.wanted(), seed=2)
+    w = {k: v * (6.0 if k.endswith("proj.weight") or k.endswith("mean.weight") else 1.0) for k, v in w.items()}
+    model = net.load(DictSource(w), torch.float32, DEV)
+    assert [type(n).__name__ for n in model.cache_needs] == ["StateNeed", "StateNeed"]
+
+    def plain(tokens):
+        x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        t = len(tokens)
+        for i in range(2):
+            p = f"model.layers.{i}."
+            h = pl.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+            x = x + (torch.cumsum(h, 0) / torch.arange(1, t + 1)[:, None]) @ w[p + "prefix_mean.weight"].T
+            h = pl.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+            x = x + pl.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        return pl.rms_norm(x, w["model.norm.weight"], 1e-5) @ w["lm_head.weight"].T
+
+    g = torch.Generator().manual_seed(1)
+    seqs = {r: torch.randint(0, vocab, (n,), generator=g).tolist() for r, n in (("a", 33), ("b", 9))}
+    refs = {r: plain(t) for r, t in seqs.items()}
+    rep = Replayer(model, 128, page_size=4)
+    assert not rep.manager.groups and len(rep.storage.states) == 2
+    for entries, end in (([("a", 0, 20), ("b", 0, 3)], []), ([("a", 20, 21), ("b", 3, 9)], ["b"]), ([("a", 21, 33)], ["a"])):
+        out = rep.step([{"id": r, "tokens": seqs[r][s:e], "want": list(range(e - s))} for r, s, e in entries], end)
+        want = torch.cat([refs[r][s:e] for r, s, e in entries])
+        assert ((out.cpu() - want).abs().amax(-1) / want.abs().amax(-1)).max() < 1e-4, entries
+    rep.manager.check()
+    # through the scheduler: greedy tokens equal the plain implementation's, whole sequence recomputed per token
+    eng = Engine(model, EngineConfig(num_blocks=8, block_size=4, max_step_tokens=16, prefill_chunk=8))
+    prompts = [seqs["a"][:11], seqs["b"][:4]]
+    reqs = [eng.add(p, SamplingParams(max_tokens=6)) for p in prompts]
+    while eng.has_work:
+        eng.step()
+    for p, r in zip(prompts, reqs):
+        seq = list(p)
+        for _ in range(6):
+            seq.append(int(plain(seq)[-1].argmax()))
+        assert r.out_tokens == seq[len(p):]
+
+
 # ------------------------------------------------------- a toy feed-forward with routing and a toy position encoding
 
 
