@@ -553,32 +553,35 @@ extern "C" int ns_silu_mul(void* out, const void* gu, int n_rows, int inter, int
 // kilobyte each; a lane then holds 32 consecutive elements of one row and writes them as 64 contiguous bytes, the four
 // lanes of a row 256.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 untile_piece;
+// kt0, n_kt: the k tiles to write out (columns 128 kt0 .. of the matrix become columns 0 .. of ``out``).
 __global__ __launch_bounds__(256) void untile_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ wt, int N, int K,
-                                                     int KT, long tiles) {
+                                                     int KT, int kt0, int n_kt, int out_stride, long tiles) {
   const int lane = threadIdx.x & 63;
-  const long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6);  // among the tiles written out
   if (tile >= tiles) return;
-  const int rt = (int)(tile / KT), kt = (int)(tile % KT);
+  const int rt = (int)(tile / n_kt), kt = kt0 + (int)(tile % n_kt);
   const int r = lane & 15, g = lane >> 4;
-  const bf16_t* src = wt + (size_t)tile * (16 * 128) + (size_t)lane * 8;
+  const bf16_t* src = wt + ((size_t)rt * KT + kt) * (16 * 128) + (size_t)lane * 8;
   untile_piece v[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const untile_piece*>(src + i * 64 * 8);
   const int row = rt * 16 + r;
   if (row >= N) return;
-  bf16_t* dst = out + (size_t)row * K + kt * 128 + g * 32;
+  bf16_t* dst = out + (size_t)row * out_stride + (kt - kt0) * 128 + g * 32;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
     if (kt * 128 + g * 32 + i * 8 < K) *reinterpret_cast<untile_piece*>(dst + i * 8) = v[i];  // K is a multiple of 8
 }
-// out: [N, K] bfloat16, contiguous, 16-byte aligned; wt: the re-laid matrix (rows padded to 16, k to 128).
-extern "C" int ns_untile_bf16(void* out, const void* wt, int N, int K, hipStream_t stream) {
+// out: bfloat16 [N, columns k0 .. k1 of the matrix] with rows out_stride elements apart, 16-byte aligned; k0 a multiple
+// of 128, k1 a multiple of 128 or K; wt: the re-laid matrix (rows padded to 16, k to 128).
+extern "C" int ns_untile_bf16(void* out, const void* wt, int N, int K, int k0, int k1, int out_stride, hipStream_t stream) {
   if (N <= 0 || K <= 0 || (K & 7) || (((uintptr_t)out | (uintptr_t)wt) & 15)) return NS_ERR_BAD_ARG;
-  const int KT = (K + 127) / 128;
-  const long tiles = (long)((N + 15) / 16) * KT;
+  if (k0 < 0 || k0 >= k1 || k1 > K || (k0 & 127) || ((k1 & 127) && k1 != K) || out_stride < k1 - k0 || (out_stride & 7)) return NS_ERR_BAD_ARG;
+  const int KT = (K + 127) / 128, kt0 = k0 / 128, n_kt = (k1 - k0 + 127) / 128;
+  const long tiles = (long)((N + 15) / 16) * n_kt;
   const long blocks = (tiles + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
-  untile_kernel<<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)wt, N, K, KT, tiles);
+  untile_kernel<<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)wt, N, K, KT, kt0, n_kt, out_stride, tiles);
   return ns_launch_status();
 }
 

@@ -278,13 +278,20 @@ class TiledWeight:
         return out
 
 
-def untile(w: TiledWeight, out: torch.Tensor) -> torch.Tensor:
-    """The matrix of ``w`` in plain rows, into ``out`` [n, k] (bfloat16, contiguous): what a library product over many rows
-    reads, made for the one product where only the re-laid copy is kept."""
+def untile(w: TiledWeight, out: torch.Tensor, k0: int = 0, k1: int | None = None) -> torch.Tensor:
+    """Columns ``k0`` to ``k1`` (all by default; ``k0`` a multiple of 128, ``k1`` one or the last column) of the matrix of
+    ``w`` in plain rows, into ``out`` [n, k1 - k0] (bfloat16, unit stride along a row): what a library product over many
+    rows reads, made for the one product where only the re-laid copy is kept."""
     _gpu(out)
-    if out.dtype != torch.bfloat16 or out.shape != (w.n, w.k) or not out.is_contiguous() or out.data_ptr() % 16 or w.k % 8:
-        raise KernelRefused(f"untile: out must be a contiguous bfloat16 [{w.n}, {w.k}], 16-byte aligned, k a multiple of 8")
-    _check(build.core().ns_untile_bf16(_ptr(out), _ptr(w.data), c_int(w.n), c_int(w.k), _stream()), "untile")
+    k1 = w.k if k1 is None else k1
+    if (out.dtype != torch.bfloat16 or out.dim() != 2 or out.shape != (w.n, k1 - k0) or out.stride(1) != 1 or out.stride(0) % 8
+            or out.data_ptr() % 16 or w.k % 8):
+        raise KernelRefused(f"untile: out must be bfloat16 [{w.n}, {k1 - k0}] with rows a multiple of 8 elements apart, 16-byte "
+                            f"aligned, and k a multiple of 8")
+    if not 0 <= k0 < k1 <= w.k or k0 % 128 or (k1 % 128 and k1 != w.k):
+        raise KernelRefused("untile: the columns start at a multiple of 128 and end at one or at the last column")
+    _check(build.core().ns_untile_bf16(_ptr(out), _ptr(w.data), c_int(w.n), c_int(w.k), c_int(k0), c_int(k1), c_int(out.stride(0)),
+                                       _stream()), "untile")
     return out
 
 

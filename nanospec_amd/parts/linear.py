@@ -30,12 +30,14 @@ STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the sha
 WIDE_HEAD_ROWS = 12  # above this many rows a wide 32-bit product (the head) is faster through the 17-to-64-row kernel
 WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
 #                    32-bit results, which the library does not give); wider products go to the library
+PLAIN_SLICE_K = 8192  # such a copy of a matrix on its way into the residual stream is made and used in slices of the inner
+#                       size no longer than this (the scratch stays small, and no product runs longer over K than the ones
+#                       that were measured)
 UNTILE_MIN_ROWS = 768  # where only the re-laid copy is kept: from this many rows on the products whose callers allow it
-#                        (``plain_copy``: q/k/v, o, gate/up) first write their matrices out in plain rows (scratch) and go to
+#                        (``plain_copy``: q/k/v, o, gate/up, down) first write their matrices out in plain rows (scratch) and go to
 #                        the library; the copy costs what 300 rows of the product cost, and the library is 1.6 to 2 times as
-#                        fast as the many-row kernel (measured for these at the 70B shape; the down-projection's comparison
-#                        is missing, so it stays with the many-row kernel).  Callers allow it in steps that are launched kernel
-#                        by kernel only: the scratch is as large as the matrix, and every captured step keeps its own.
+#                        fast as the many-row kernel (measured at the 70B shape).  Callers allow it in steps that are launched
+#                        kernel by kernel only: the scratch is as large as the matrix, and every captured step keeps its own.
 
 
 class IntoResidual:
@@ -97,8 +99,22 @@ class LinearWeight:
         r = link.resid
         plain_t = self._plain_t
         if (plain_t is None and plain_copy and self.tiled is not None and m >= UNTILE_MIN_ROWS and x.dtype == torch.bfloat16
-                and ops.tiled_takes(x[:1], self.k)):
-            plain_t = ops.untile(self.tiled, take((self.n, self.k), self.dtype)).t()  # only the re-laid copy is kept, many rows
+                and ops.tiled_takes(x[:1], self.k)):  # only the re-laid copy is kept, many rows
+            if self.k > PLAIN_SLICE_K and r.dtype == torch.bfloat16 and r.shape == (m, self.n) and r.is_contiguous():
+                # a long inner size in slices: the stream in 32-bit takes every slice's product as the library adds it
+                # (32-bit sums, 32-bit addend and result) and is rounded once at the end, as one product would be
+                slices = -(-self.k // PLAIN_SLICE_K)
+                width = -(-self.k // (128 * slices)) * 128
+                acc = take((m, self.n), torch.float32)
+                acc.copy_(r)
+                plain = take((self.n, width), self.dtype)
+                for k0 in range(0, self.k, width):
+                    k1 = min(self.k, k0 + width)
+                    piece = ops.untile(self.tiled, plain[:, : k1 - k0], k0, k1)
+                    torch.addmm(acc, x[:, k0:k1], piece.t(), out_dtype=torch.float32, out=acc)
+                r.copy_(acc)
+                return ops.Added()
+            plain_t = ops.untile(self.tiled, take((self.n, self.k), self.dtype)).t()
         if (m > ops.SKINNY_MAX_ROWS and plain_t is not None and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16
                 and r.shape == (m, self.n) and r.is_contiguous()):
             # many rows: the library's product takes the stream as its addend, resid = resid + x @ W^T summed in 32-bit and
@@ -140,7 +156,7 @@ class LinearWeight:
             return torch.matmul(x, self._plain_t) if out is None else torch.matmul(x, self._plain_t, out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
-        if m >= UNTILE_MIN_ROWS and not out_f32 and plain_copy:  # only the tiled layout is kept, many rows: a plain copy for this one product
+        if m >= UNTILE_MIN_ROWS and not out_f32 and plain_copy and self.k <= PLAIN_SLICE_K:  # only the tiled layout is kept, many rows: a plain copy for this one product
             plain = arena.take((self.n, self.k), self.dtype) if arena is not None else torch.empty((self.n, self.k), dtype=self.dtype, device=x.device)
             return torch.matmul(x, ops.untile(self.tiled, plain).t(), out=out)
         if m > ops.WIDE_TALL_ROWS:  # ... fewer: blocks of 128 rows through the hand-written kernel

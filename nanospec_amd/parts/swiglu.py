@@ -41,8 +41,8 @@ class SwiGLU:
     def forward(self, ctx, x, out: torch.Tensor | None = None, residual=None):
         act = self.gate_up(ctx, x, out=ctx.arena.take((x.shape[0], self.spec.intermediate), x.dtype))
         if residual is not None:
-            return self.down.into_residual(act, residual, arena=ctx.arena)
-        return self.down(act, out=out, arena=ctx.arena)
+            return self.down.into_residual(act, residual, arena=ctx.arena, plain_copy=not ctx.captured)
+        return self.down(act, out=out, arena=ctx.arena, plain_copy=not ctx.captured)
 
 
 registry.register("ffn", "swiglu", SwiGLU)

@@ -550,6 +550,13 @@ def test_untile_gives_the_matrix_back(n, k):
     assert bool((guard[0] == 7).all()) and bool((guard[-1] == 7).all())
     with pytest.raises(ops.KernelRefused):
         ops.untile(ops.TiledWeight(w), torch.empty(n, k + 8, dtype=torch.bfloat16, device=DEV))
+    if k > 128:  # a range of columns, into rows that are further apart than they are long
+        k0, k1 = 128, k if k < 384 else 384
+        wide = torch.full((n, k1 - k0 + 16), 7.0, dtype=torch.bfloat16, device=DEV)
+        ops.untile(ops.TiledWeight(w), wide[:, : k1 - k0], k0, k1)
+        assert torch.equal(wide[:, : k1 - k0], w[:, k0:k1]) and bool((wide[:, k1 - k0 :] == 7).all())
+        with pytest.raises(ops.KernelRefused):
+            ops.untile(ops.TiledWeight(w), wide[:, : k1 - k0 - 8], k0 + 8, k1)
 
 
 def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0,
