@@ -97,10 +97,14 @@ class LinearWeight:
             if ws is not None:
                 return ops.linear_wide(x, self.tiled, workspace=ws, ksplit=ksplit, nt=nt, defer=True)
         r = link.resid
+        # many rows: the library's product takes the stream as its addend, resid = resid + x @ W^T summed in 32-bit and
+        # rounded once, so the norm after it reads one tensor instead of two and writes one instead of two
+        library = (m > ops.SKINNY_MAX_ROWS and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16 and r.shape == (m, self.n)
+                   and r.is_contiguous())
         plain_t = self._plain_t
-        if (plain_t is None and plain_copy and self.tiled is not None and m >= UNTILE_MIN_ROWS and x.dtype == torch.bfloat16
+        if (library and plain_t is None and plain_copy and self.tiled is not None and m >= UNTILE_MIN_ROWS
                 and ops.tiled_takes(x[:1], self.k)):  # only the re-laid copy is kept, many rows
-            if self.k > PLAIN_SLICE_K and r.dtype == torch.bfloat16 and r.shape == (m, self.n) and r.is_contiguous():
+            if self.k > PLAIN_SLICE_K:
                 # a long inner size in slices: the stream in 32-bit takes every slice's product as the library adds it
                 # (32-bit sums, 32-bit addend and result) and is rounded once at the end, as one product would be
                 slices = -(-self.k // PLAIN_SLICE_K)
@@ -115,10 +119,7 @@ class LinearWeight:
                 r.copy_(acc)
                 return ops.Added()
             plain_t = ops.untile(self.tiled, take((self.n, self.k), self.dtype)).t()
-        if (m > ops.SKINNY_MAX_ROWS and plain_t is not None and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16
-                and r.shape == (m, self.n) and r.is_contiguous()):
-            # many rows: the library's product takes the stream as its addend, resid = resid + x @ W^T summed in 32-bit and
-            # rounded once, so the norm after it reads one tensor instead of two and writes one instead of two
+        if library and plain_t is not None:
             r.addmm_(x, plain_t)
             return ops.Added()
         out = link.x_next if link.x_next is not None else take((m, self.n), x.dtype)
