@@ -7,7 +7,8 @@ step function, captured graphs, sampling).  The benchmark decodes from context 2
 linearly with the context, so K timed steps (after W untimed ones) are taken as a window centred on context 3,072,
 the mean of 2,048..4,096, and stand for the whole run; with K >= 2,048 the whole run is timed (prompts of 2,048
 random token ids, then 2,048 decode steps).  ``metric`` and ``config`` name the contexts that were timed.  ``points``
-holds the same at batch 1 and 64 (windows of at most 256 steps), and the new tokens per second of 32 requests served by
+holds the same at batch 1 and 64 (windows of at most 256 steps), one request with a prompt of 128 tokens and 256 new tokens
+timed as a whole (``decode_b1_ctx128``: the workload of the one figure that the reference publishes), and the new tokens per second of 32 requests served by
 continuous batching at the Llama-3.2-1B shape (prompts of 16 to 1,024 tokens in portions of 512, 128 new tokens each);
 ``points_roofline_frac`` holds their fractions of the memory roofline (for the serving run: of what memory and matrix units
 need together).  ``prefill`` is one step of 2,048 prompt tokens of one request; ``roofline`` is the bytes a decode
@@ -119,6 +120,36 @@ def prefill_run(model, cfg, n_tokens: int, block_size: int, reps: int = 3, porti
         if i and (best is None or dt < best):
             best = dt  # the first pass warms the library's kernel selection
     del rep
+    torch.cuda.empty_cache()
+    return best
+
+
+def short_run(model, cfg, prompt_len: int, new_tokens: int, block_size: int, reps: int = 2):
+    """One request at a time, a short prompt and ``new_tokens`` greedy tokens, timed from ``add`` to the last token with the
+    prompt's step included (the reference's own workload and clock: bench/run.py:162-172, batch 1, 256 new tokens after a
+    short chat prompt).  -> seconds of the best pass; the first pass captures the graphs and is not timed."""
+    import torch
+
+    from nanospec_amd import Engine, EngineConfig, SamplingParams
+
+    total = prompt_len + new_tokens + 2
+    eng = Engine(model, EngineConfig(num_blocks=-(-total // block_size) + 4, block_size=block_size, max_admit=1, max_running=1,
+                                     max_step_tokens=2048, prefill_chunk=2048, max_seq_len=total + block_size))
+    g = torch.Generator().manual_seed(11)
+    best = None
+    for i in range(reps + 1):
+        prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        req = eng.add(prompt, SamplingParams(max_tokens=new_tokens))
+        while eng.has_work:
+            eng.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert len(req.out_tokens) == new_tokens
+        if i and (best is None or dt < best):
+            best = dt
+    del eng
     torch.cuda.empty_cache()
     return best
 
@@ -248,6 +279,13 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * k / d, 1)
             nbytes = weight_bytes(cfg, esize) + b * (c0 + c1 - 1) / 2 * kv_bytes_per_token(cfg, esize)
             points_frac[f"decode_b{b}"] = round(nbytes / (d / k) / 1e9 / HBM_GBPS, 4)
+
+        # the reference's own published workload (README.md:72-76: 137 tok/s on an H100): one request, a short prompt, 256 new
+        # tokens, the clock around the whole request
+        d = short_run(model, cfg, 128, 256, block)
+        points["decode_b1_ctx128"] = round(256 / d, 1)
+        nbytes = weight_bytes(cfg, esize) + (128 + 128) * kv_bytes_per_token(cfg, esize)
+        points_frac["decode_b1_ctx128"] = round(nbytes / (d / 256) / 1e9 / HBM_GBPS, 4)
 
     if not a.no_points and a.shape == "8b" and not a.layers:
         # the serving workload beside the headline: 32 requests through the Llama-3.2-1B shape, continuous batching with

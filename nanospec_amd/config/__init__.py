@@ -1,5 +1,5 @@
-from .llama import LlamaConfig
 from .registry import architectures, load_config, register_architecture, resolve
+from .llama import LlamaConfig  # (importing an architecture's module registers it)
 from .spec import (AttentionSpec, LayerCall, ModelSpec, NoPositionSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec,
                    SwiGLUSpec)
 

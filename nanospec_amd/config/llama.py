@@ -8,6 +8,7 @@ from __future__ import annotations
 import math
 from dataclasses import dataclass, field
 
+from .registry import register_architecture
 from .spec import AttentionSpec, LayerCall, ModelSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
 
 _LLAMA3_KEYS = ("factor", "low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
@@ -157,3 +158,11 @@ class LlamaConfig:
             tie_head=self.tie_word_embeddings,
             eos_token_ids=self.eos_token_ids,
         )
+
+
+def _build(cfg: dict, generation_cfg: dict | None):
+    config = LlamaConfig.from_hf(cfg, generation_cfg)
+    return config, config.model_spec()
+
+
+register_architecture("LlamaForCausalLM", _build, model_type="llama")

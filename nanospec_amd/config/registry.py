@@ -3,7 +3,8 @@
 An entry is a function ``(config.json dict, generation_config.json dict or None) -> (typed
 configuration, ModelSpec)``.  Everything downstream (weights, parts, cache, engine) works from the
 ``ModelSpec`` alone, so another architecture is one typed configuration, its ``model_spec()`` and
-one ``register_architecture`` call.
+one ``register_architecture`` call, made by the architecture's own module when it is imported (``config/llama.py``
+does so; nothing here names an architecture).
 """
 
 from __future__ import annotations
@@ -12,8 +13,7 @@ import json
 from pathlib import Path
 from typing import Callable
 
-from .llama import LlamaConfig
-from .spec import ModelSpec
+from .spec import ModelSpec  # noqa: F401  (what an entry returns)
 
 _ARCHITECTURES: dict[str, Callable] = {}
 _MODEL_TYPES: dict[str, str] = {}  # config.json model_type -> architecture, for files without `architectures`
@@ -52,11 +52,3 @@ def load_config(folder):
     gen_path = folder / "generation_config.json"
     gen = json.loads(gen_path.read_text()) if gen_path.is_file() else None
     return resolve(cfg, gen)
-
-
-def _llama(cfg: dict, generation_cfg: dict | None):
-    config = LlamaConfig.from_hf(cfg, generation_cfg)
-    return config, config.model_spec()
-
-
-register_architecture("LlamaForCausalLM", _llama, model_type="llama")

@@ -26,15 +26,18 @@ class RMSNormSpec:
 
 @dataclass(frozen=True)
 class RopeSpec:
-    """Rotary position encoding over the first ``rotary_dim`` elements of a head; element j is
-    paired with j + rotary_dim/2.  ``scaling`` is None or the llama3 frequency scaling as
-    (factor, low_freq_factor, high_freq_factor, original_max_position_embeddings)."""
+    """Rotary position encoding over the first ``rotary_dim`` elements of a head; pair j is elements j and
+    j + rotary_dim/2 (``interleaved``: 2j and 2j + 1).  ``scaling`` is None or the llama3 frequency scaling as
+    (factor, low_freq_factor, high_freq_factor, original_max_position_embeddings).  ``cos_sin_factor`` multiplies
+    cosine and sine."""
 
     kind: ClassVar[str] = "rope"
     rotary_dim: int
     theta: float
     scaling: tuple[float, float, float, int] | None = None
     max_positions: int | None = None  # None = unbounded
+    interleaved: bool = False
+    cos_sin_factor: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -108,6 +111,10 @@ class ModelSpec:
     head_name: str  # tensor name of the [vocab, hidden] output matrix
     tie_head: bool  # a missing head tensor is the embedding table
     eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+    # what an architecture may do at the two ends of the stack; the defaults do nothing and launch nothing
+    embed_scale: float = 1.0  # the embedding rows are multiplied by this as they enter the stream
+    logit_scale: float = 1.0  # the head's 32-bit logits are multiplied by this ...
+    logit_softcap: float = 0.0  # ... and then, if > 0, become softcap * tanh(logit / softcap)
 
     def __post_init__(self) -> None:
         for pos, call in enumerate(self.run_order):

@@ -2,26 +2,53 @@
 // write of keys and values into cache pages, and SiLU(gate)*up.  One template per kernel over the
 // storage type (float or bfloat16); all arithmetic is 32-bit.
 #include "common.h"
+#include "rope.h"
 
 // ------------------------------------------------------------------------------------------------
-// Embedding: out[i, :] = table[ids[i], :]                     (reference: model/llama.py:221)
+// Embedding: out[i, :] = table[ids[i], :] (* scale, rounded once)      (reference: model/llama.py:221; a scale of 1
+//                                                                       copies the row as it is)
 // ------------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void embed_kernel(T* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids, int hidden) {
+__global__ void embed_kernel(T* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids, int hidden, float scale) {
   const int row = blockIdx.x;
   const T* src = table + (size_t)ids[row] * hidden;
   T* dst = out + (size_t)row * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  if (scale == 1.f)
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  else
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_f<T>(to_f(src[i]) * scale);
 }
 
-extern "C" int ns_embed(void* out, const void* table, const int* ids, int n_tokens, int hidden, int dtype, hipStream_t stream) {
+extern "C" int ns_embed(void* out, const void* table, const int* ids, int n_tokens, int hidden, float scale, int dtype,
+                        hipStream_t stream) {
   if (n_tokens <= 0 || hidden <= 0) return NS_ERR_BAD_ARG;
   if (dtype == NS_DTYPE_F32)
-    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)out, (const float*)table, ids, hidden);
+    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)out, (const float*)table, ids, hidden, scale);
   else if (dtype == NS_DTYPE_BF16)
-    embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)table, ids, hidden);
+    embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)table, ids, hidden, scale);
   else
     return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// 32-bit logits in place: l = l * scale; with a cap > 0 then l = cap * tanh(l / cap).  For architectures whose head
+// ends in a scale or a soft cap; the Llama head has neither and never launches this.
+// ------------------------------------------------------------------------------------------------
+__global__ void logit_transform_kernel(float* __restrict__ logits, int vocab, int stride, float scale, float cap) {
+  float* row = logits + (size_t)blockIdx.y * stride;
+  const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < vocab; i += gridDim.x * blockDim.x) {
+    float v = row[i] * scale;
+    if (cap > 0.f) v = cap * tanhf(v * inv_cap);
+    row[i] = v;
+  }
+}
+
+extern "C" int ns_logit_transform(float* logits, int rows, int vocab, int stride, float scale, float cap, hipStream_t stream) {
+  if (rows <= 0 || rows > 65535 || vocab <= 0 || stride < vocab || cap < 0.f) return NS_ERR_BAD_ARG;
+  const int bx = (vocab + 1023) / 1024 < 64 ? (vocab + 1023) / 1024 : 64;
+  logit_transform_kernel<<<dim3(bx, rows), 256, 0, stream>>>(logits, vocab, stride, scale, cap);
   return ns_launch_status();
 }
 
@@ -251,27 +278,24 @@ template <typename T>
 __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                                const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
                                const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                               int heads, int kv_heads, int hd, int rot, int page_size, int write_kv) {
+                               int heads, int kv_heads, int hd, RopeForm form, int page_size, int write_kv) {
   extern __shared__ float cs[];  // cos[half] | sin[half] of this token's angles
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (size_t)t * row_stride;
-  const int half = rot / 2;
-  const float fpos = (float)pos;
-  for (int j = threadIdx.x; j < half; j += blockDim.x) {
-    const float ang = fpos * inv_freq[j];
-    cs[j] = cosf(ang);
-    cs[half + j] = sinf(ang);
-  }
+  const int rot = form.rot, half = rot / 2;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) rope_cos_sin(form, pos, inv_freq[j], cs[j], cs[half + j]);
   __syncthreads();
   // q heads, in place
   for (int e = threadIdx.x; e < heads * half; e += blockDim.x) {
     const int h = e / half, j = e - h * half;
-    const float c = cs[j], s = cs[half + j];
+    int d1, d2;
+    rope_pair_channels(form, j, d1, d2);
     T* p = row + h * hd;
-    const float a = to_f(p[j]), b = to_f(p[j + half]);
-    p[j] = from_f<T>(a * c - b * s);
-    p[j + half] = from_f<T>(b * c + a * s);
+    float a, b;
+    rope_turn(to_f(p[d1]), to_f(p[d2]), cs[j], cs[half + j], a, b);
+    p[d1] = from_f<T>(a);
+    p[d2] = from_f<T>(b);
   }
   if (!write_kv) return;
   const int page = block_table[(size_t)token_req[t] * table_stride + pos / page_size];
@@ -280,52 +304,48 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, int row_stride, const int* _
   const T* vrow = krow + kv_heads * hd;
   T* kdst = k_cache + (size_t)page * kv_heads * page_size * hd + (size_t)off * hd;
   T* vdst = v_cache + (size_t)page * kv_heads * hd * page_size + off;
-  for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x) {
-    const int h = e / hd, d = e - h * hd;
-    float kv;
-    if (d < rot) {
-      const int j = d < half ? d : d - half;
-      const float c = cs[j], s = cs[half + j];
-      const float a = to_f(krow[h * hd + j]), b = to_f(krow[h * hd + j + half]);
-      kv = d < half ? a * c - b * s : b * c + a * s;
-    } else {
-      kv = to_f(krow[e]);
-    }
-    kdst[(size_t)h * page_size * hd + d] = from_f<T>(kv);
-    vdst[(size_t)e * page_size] = vrow[e];
+  for (int e = threadIdx.x; e < kv_heads * half; e += blockDim.x) {  // the rotary pairs of k
+    const int h = e / half, j = e - h * half;
+    int d1, d2;
+    rope_pair_channels(form, j, d1, d2);
+    float a, b;
+    rope_turn(to_f(krow[h * hd + d1]), to_f(krow[h * hd + d2]), cs[j], cs[half + j], a, b);
+    kdst[(size_t)h * page_size * hd + d1] = from_f<T>(a);
+    kdst[(size_t)h * page_size * hd + d2] = from_f<T>(b);
   }
+  const int plain = hd - rot;  // channels of a head beyond the rotary part
+  for (int e = threadIdx.x; e < kv_heads * plain; e += blockDim.x) {
+    const int h = e / plain, d = rot + e - h * plain;
+    kdst[(size_t)h * page_size * hd + d] = krow[h * hd + d];
+  }
+  for (int e = threadIdx.x; e < kv_heads * hd; e += blockDim.x) vdst[(size_t)e * page_size] = vrow[e];
 }
 
 // The same with 16-byte accesses for q and k (values still go element by element into their transposed page): a
-// thread takes V consecutive channels j.. of the first half and their partners j + rot/2.  For rot/2, hd - rot and
-// the row stride multiples of V elements and 16-byte aligned buffers.
+// thread takes V consecutive channels j.. of the first half and their partners j + rot/2.  For the half-split pairing,
+// rot/2, hd - rot and the row stride multiples of V elements and 16-byte aligned buffers.
 template <typename T>
 __global__ void rope_kv_vec_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                                    const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
                                    const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                   int heads, int kv_heads, int hd, int rot, int page_size, int write_kv) {
+                                   int heads, int kv_heads, int hd, RopeForm form, int page_size, int write_kv) {
   constexpr int V = 16 / sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(V)));
   extern __shared__ float cs[];  // cos[half] | sin[half] of this token's angles
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (size_t)t * row_stride;
-  const int half = rot / 2;
-  const float fpos = (float)pos;
-  for (int j = threadIdx.x; j < half; j += blockDim.x) {
-    const float ang = fpos * inv_freq[j];
-    cs[j] = cosf(ang);
-    cs[half + j] = sinf(ang);
-  }
+  const int rot = form.rot, half = rot / 2;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) rope_cos_sin(form, pos, inv_freq[j], cs[j], cs[half + j]);
   __syncthreads();
   const int per_head = half / V;  // vector pairs per head
   auto turn = [&](const vec_t a, const vec_t b, int j, vec_t& lo, vec_t& hi) {
 #pragma unroll
     for (int e = 0; e < V; ++e) {
-      const float c = cs[j + e], s = cs[half + j + e];
-      const float x = to_f(a[e]), y = to_f(b[e]);
-      lo[e] = from_f<T>(x * c - y * s);
-      hi[e] = from_f<T>(y * c + x * s);
+      float x, y;
+      rope_turn(to_f(a[e]), to_f(b[e]), cs[j + e], cs[half + j + e], x, y);
+      lo[e] = from_f<T>(x);
+      hi[e] = from_f<T>(y);
     }
   };
   for (int u = threadIdx.x; u < heads * per_head; u += blockDim.x) {
@@ -384,33 +404,34 @@ __global__ void rope_kv_vec_kernel(T* __restrict__ qkv, int row_stride, const in
 
 extern "C" int ns_rope_kv_write(void* qkv, int row_stride, const int* positions, const int* token_req,
                                 const int* block_table, int table_stride, const float* inv_freq, void* k_cache,
-                                void* v_cache, int n_tokens, int heads, int kv_heads, int hd, int rot, int page_size,
-                                int write_kv, int dtype, hipStream_t stream) {
+                                void* v_cache, int n_tokens, int heads, int kv_heads, int hd, int rot, int interleaved,
+                                float factor, int page_size, int write_kv, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || rot < 0 || rot > hd || (rot & 1) || page_size <= 0)
     return NS_ERR_BAD_ARG;
+  const RopeForm form = {rot, interleaved ? 1 : 0, factor};
   const int work = heads * (rot / 2) > kv_heads * hd ? heads * (rot / 2) : kv_heads * hd;
   const int threads = work >= 1024 ? 1024 : work >= 512 ? 512 : 256;
   const int vlen = dtype == NS_DTYPE_F32 ? 4 : 8;
   const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0 && row_stride % vlen == 0 && (rot / 2) % vlen == 0 &&
-                       (hd - rot) % vlen == 0 && hd % vlen == 0 && rot > 0;
+                       (hd - rot) % vlen == 0 && hd % vlen == 0 && rot > 0 && !interleaved;
   if (aligned) {
     const int vthreads = threads >= 512 ? 256 : threads;
     if (dtype == NS_DTYPE_F32)
       rope_kv_vec_kernel<float><<<n_tokens, vthreads, (size_t)(rot + 2) * sizeof(float), stream>>>((float*)qkv, row_stride, positions, token_req, block_table, table_stride,
-                                                          inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
+                                                          inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, form, page_size, write_kv);
     else if (dtype == NS_DTYPE_BF16)
       rope_kv_vec_kernel<bf16_t><<<n_tokens, vthreads, (size_t)(rot + 2) * sizeof(float), stream>>>((bf16_t*)qkv, row_stride, positions, token_req, block_table, table_stride,
-                                                           inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
+                                                           inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, form, page_size, write_kv);
     else
       return NS_ERR_UNSUPPORTED;
     return ns_launch_status();
   }
   if (dtype == NS_DTYPE_F32)
     rope_kv_kernel<float><<<n_tokens, threads, (size_t)(rot + 2) * sizeof(float), stream>>>((float*)qkv, row_stride, positions, token_req, block_table, table_stride,
-                                                        inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
+                                                        inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, form, page_size, write_kv);
   else if (dtype == NS_DTYPE_BF16)
     rope_kv_kernel<bf16_t><<<n_tokens, threads, (size_t)(rot + 2) * sizeof(float), stream>>>((bf16_t*)qkv, row_stride, positions, token_req, block_table, table_stride,
-                                                         inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, rot, page_size, write_kv);
+                                                         inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, form, page_size, write_kv);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
@@ -428,7 +449,8 @@ __global__ __launch_bounds__(256) void rope_kv_partial_kernel(bf16_t* __restrict
                                                               const int* __restrict__ token_req, const int* __restrict__ block_table,
                                                               int table_stride, const float* __restrict__ inv_freq,
                                                               bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int heads,
-                                                              int kv_heads, int hd, int rot, int page_size, int write_kv) {
+                                                              int kv_heads, int hd, RopeForm form, int page_size, int write_kv) {
+  const int rot = form.rot;
   const int m = blockIdx.x;
   const int u = blockIdx.y * blockDim.x + threadIdx.x;  // (tile, pair)
   const int tiles_per_head = hd / 16;
@@ -450,13 +472,10 @@ __global__ __launch_bounds__(256) void rope_kv_partial_kernel(bf16_t* __restrict
   int d1, d2;
   if (rotary) {
     const int j = jt * 8 + p;
-    const float ang = (float)pos * inv_freq[j];
-    const float c = cosf(ang), sn = sinf(ang);
-    const float a = x1, b = x2;
-    x1 = a * c - b * sn;
-    x2 = b * c + a * sn;
-    d1 = j;
-    d2 = j + rot / 2;
+    float c, sn;
+    rope_cos_sin(form, pos, inv_freq[j], c, sn);
+    rope_turn(x1, x2, c, sn, x1, x2);
+    rope_pair_channels(form, j, d1, d2);
   } else {
     d1 = (is_v ? 0 : rot) + (jt - rot_tiles) * 16 + p;
     d2 = d1 + 8;
@@ -482,16 +501,16 @@ __global__ __launch_bounds__(256) void rope_kv_partial_kernel(bf16_t* __restrict
 
 extern "C" int ns_rope_kv_partial(void* q_out, int q_stride, const float* partial, int ksplit, int M, int N, const int* positions,
                                   const int* token_req, const int* block_table, int table_stride, const float* inv_freq,
-                                  void* k_cache, void* v_cache, int heads, int kv_heads, int hd, int rot, int page_size, int write_kv,
-                                  hipStream_t stream) {
+                                  void* k_cache, void* v_cache, int heads, int kv_heads, int hd, int rot, int interleaved,
+                                  float factor, int page_size, int write_kv, hipStream_t stream) {
   if (M <= 0 || M > 65535 || ksplit < 1 || heads <= 0 || kv_heads <= 0 || hd <= 0 || (hd & 15) || rot < 0 || rot > hd || (rot & 15) ||
       page_size <= 0 || N != (heads + 2 * kv_heads) * hd || q_stride < heads * hd)
     return NS_ERR_BAD_ARG;
   const int units = N / 2;  // pairs of columns per token
   dim3 grid(M, (units + 255) / 256);
   rope_kv_partial_kernel<<<grid, 256, 0, stream>>>((bf16_t*)q_out, q_stride, partial, ksplit, M, N, positions, token_req, block_table,
-                                                   table_stride, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, rot,
-                                                   page_size, write_kv);
+                                                   table_stride, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd,
+                                                   RopeForm{rot, interleaved ? 1 : 0, factor}, page_size, write_kv);
   return ns_launch_status();
 }
 

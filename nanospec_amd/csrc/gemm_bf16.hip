@@ -15,6 +15,7 @@
 // (reference: model/llama.py:195); rotation and cache write for the stacked q/k/v matrix.
 // (reference for the products themselves: the nn.Linear calls of model/llama.py:175,184,195,286)
 #include "common.h"
+#include "rope.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
@@ -32,8 +33,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 // and 7 of the other.
 
 // What the q/k/v epilogue needs: the rows of the stacked [q; k; v] matrix were permuted at load time so that a
-// workgroup's 16 rows are, for the rotary part of a q or k head, 8 channels j and their partners j + rot/2, and
-// otherwise 16 consecutive channels.  The epilogue rotates (angle = position * inv_freq[j], 32-bit), writes q into
+// workgroup's 16 rows are, for the rotary part of a q or k head, the first channels of 8 pairs j and then their second
+// channels (rope.h: j and j + rot/2, or 2j and 2j + 1), and otherwise 16 consecutive channels.  The epilogue rotates
+// (rope.h), writes q into
 // the attention input, k into its K page slot and v into the transposed V page
 // (reference: model/llama.py:175-183; kv/cache.py:23-26).
 struct RopeKvParams {
@@ -44,6 +46,7 @@ struct RopeKvParams {
   bf16_t* k_cache;         // [pages, kv_heads, page, hd]
   bf16_t* v_cache;         // [pages, kv_heads, hd, page]
   int table_stride, heads, kv_heads, hd, rot, page_size, write_kv;
+  RopeForm form;           // rot again, the pairing and the factor on cosine and sine
 };
 
 // How a product can take over the work of the norm kernels around it (reference for the norm: model/llama.py:86-95, for
@@ -205,7 +208,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
     const bool is_q = gh < rk.heads, is_v = gh >= rk.heads + rk.kv_heads;
     const int rot_tiles = is_v ? 0 : rk.rot / 16;
     const bool rotary = jt < rot_tiles;
-    const int half = rk.rot / 2;
     for (int e = threadIdx.x; e < M * 8; e += WAVES * 64) {
       const int m = e >> 3, p = e & 7;
       const int mt = m >> 4, mr = m & 15;
@@ -224,13 +226,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
       int d1, d2;
       if (rotary) {
         const int j = jt * 8 + p;
-        const float ang = (float)rk.positions[m] * rk.inv_freq[j];
-        const float c = cosf(ang), sn = sinf(ang);
-        const float a = x1, b = x2;
-        x1 = a * c - b * sn;
-        x2 = b * c + a * sn;
-        d1 = j;
-        d2 = j + half;
+        float c, sn;
+        rope_cos_sin(rk.form, rk.positions[m], rk.inv_freq[j], c, sn);
+        rope_turn(x1, x2, c, sn, x1, x2);
+        rope_pair_channels(rk.form, j, d1, d2);
       } else {
         d1 = rk.rot * (is_v ? 0 : 1) + (jt - rot_tiles) * 16 + p;
         d2 = d1 + 8;
@@ -409,14 +408,15 @@ extern "C" int ns_gemm_resid_norm_bf16(void* resid, void* x_next, void* ssq_out,
 extern "C" int ns_gemm_qkv_rope_bf16(void* q_out, const void* x, const void* wt, int M, int K, int x_stride, int q_stride,
                                      const int* positions, const int* token_req, const int* block_table, int table_stride,
                                      const float* inv_freq, void* k_cache, void* v_cache, int heads, int kv_heads, int hd,
-                                     int rot, int page_size, int write_kv, int waves, const float* ssq_in, int parts_in,
-                                     int norm_dim, float eps, hipStream_t stream) {
+                                     int rot, int interleaved, float factor, int page_size, int write_kv, int waves,
+                                     const float* ssq_in, int parts_in, int norm_dim, float eps, hipStream_t stream) {
   if (M > 16 || hd % 16 || rot % 16 || rot > hd || heads <= 0 || kv_heads <= 0 || page_size <= 0 || q_stride < heads * hd)
     return NS_ERR_BAD_ARG;
   RopeKvParams rk;
   rk.positions = positions; rk.token_req = token_req; rk.block_table = block_table; rk.inv_freq = inv_freq;
   rk.k_cache = (bf16_t*)k_cache; rk.v_cache = (bf16_t*)v_cache; rk.table_stride = table_stride; rk.heads = heads;
   rk.kv_heads = kv_heads; rk.hd = hd; rk.rot = rot; rk.page_size = page_size; rk.write_kv = write_kv;
+  rk.form = RopeForm{rot, interleaved ? 1 : 0, factor};
   NormLink nl = {};
   nl.ssq_in = ssq_in; nl.parts_in = parts_in; nl.inv_dim = norm_dim > 0 ? 1.f / (float)norm_dim : 0.f; nl.eps = eps;
   const int N = (heads + 2 * kv_heads) * hd;

@@ -22,7 +22,8 @@ class Arena:
         self._chunks: list[torch.Tensor] = []
         self._typed: dict = {}  # (chunk, dtype) -> the chunk seen as that type
         self._cur, self._off = -1, 0
-        self._high = 0  # bytes one step needed at most, over all chunks
+        self.high_water = 0  # the most bytes that were in use at once since the arena was made (tails of chunks that a buffer
+        #                      did not fit into count as used: one chunk of this size holds the same sequence of buffers)
         if nbytes:
             self._chunks.append(torch.empty(nbytes, dtype=torch.uint8, device=device))
             self._cur = 0
@@ -51,7 +52,14 @@ class Arena:
         first = self._off // esize
         out = typed[first : first + count].view(shape)
         self._off += need
+        used = self._off + sum(c.numel() for c in self._chunks[: self._cur])
+        if used > self.high_water:
+            self.high_water = used
         return out
+
+    @property
+    def capacity(self) -> int:
+        return sum(c.numel() for c in self._chunks)
 
     def mark(self) -> tuple[int, int]:
         return self._cur, self._off

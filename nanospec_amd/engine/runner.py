@@ -22,7 +22,7 @@ from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage
 from ..kernels import ops
 from .arena import Arena
-from .context import CHUNK_TILE, BatchLayout, StepContext, count_tiles, fill_batch
+from .context import BatchLayout, StepContext, fill_batch
 
 # reference: engine/graphs.py:22 (powers of two up to 64).  48 and 96 besides: the products' cost goes by 16 rows at a time
 # between 17 and 128 rows, so 40 requests padded to 64 rows pay for a quarter more than padded to 48.  Above 128 rows
@@ -46,13 +46,15 @@ class StepEntry:
 MIXED_PORTIONS = 4
 MIXED_TOKEN_STEP = 64
 MIXED_MAX_TOKENS = 1024
-MAX_GRAPHS = 96  # captured steps kept; the one not used for longest goes first
+MAX_GRAPHS = 96  # captured steps kept; the one not used for longest goes first.  What a captured step holds for itself is
+#                   small (its batch buffer on both sides and its samples); the intermediates of all of them lie in one
+#                   shared arena, see ``ModelRunner._arena_for``
 
 
 class _StepGraph:
     """One captured step of a fixed shape: ``rows`` requests that bring one token each and up to ``portions`` requests
-    that bring ``chunk`` tokens together; a static batch buffer, an arena of fixed addresses, logits and samples for
-    ``rows + portions`` wanted places.  What a step does not fill is padding: pad rows and pad tokens belong to the
+    that bring ``chunk`` tokens together; a static batch buffer, fixed addresses in the arena that all captured steps share
+    (they replay one after another on one stream), logits and samples for ``rows + portions`` wanted places.  What a step does not fill is padding: pad rows and pad tokens belong to the
     runner's pad request (position 0 of a page nobody reads), tiles without tokens, wanted rows that nobody reads."""
 
     def __init__(self, runner: "ModelRunner", rows: int, chunk: int, width: int) -> None:
@@ -61,13 +63,13 @@ class _StepGraph:
         n_groups = len(runner.manager.groups)
         self.n_reqs = rows + self.portions + (1 if chunk else 0)  # the last one owns the pad tokens
         self.n_want = rows + self.portions
-        tiles = -(-chunk // CHUNK_TILE) + self.portions if chunk else 0  # every portion may end in a tile that is not full
-        self.layout = BatchLayout(rows + chunk, self.n_reqs, self.n_want, tiles, rows, n_groups, width, n_patch=rows, n_sample=self.n_want)
+        plans = [(p, p.shape_captured(rows, chunk, self.portions)) for p in runner.plans]
+        self.layout = BatchLayout(rows + chunk, self.n_reqs, self.n_want, n_groups, width, n_patch=rows, n_sample=self.n_want, plans=plans)
         dev = runner.device
         self.dev_buf = torch.zeros(self.layout.total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
         self.host_np = self.host.numpy()
-        self.arena = Arena(dev)  # grows during the warm-up run, then stays as it is
+        self.arena: Arena | None = None  # the captured steps' shared arena, given at capture
         self.logits: torch.Tensor | None = None
         self.sampled = torch.zeros((3, self.n_want), dtype=torch.int32, device=dev)  # what the captured sampling kernel writes
         self.graph = None
@@ -80,9 +82,9 @@ class _StepGraph:
         f = opts[:3].view(torch.float32)
         return f[0], f[1], f[2], opts[3]
 
-    def context(self, runner) -> StepContext:
-        return StepContext(self.layout, self.dev_buf, self.arena, link_norms=runner.link_norms, max_position=0,
-                           max_kv_len=self.width * runner.page_size, captured=True)
+    def context(self, runner, arena) -> StepContext:
+        return StepContext(self.layout, self.dev_buf, arena, link_norms=runner.link_norms, max_position=0,
+                           max_kv_len=self.width * runner.page_size, captured=True, pad_slot=runner.manager.get(PAD_REQUEST).slot)
 
 
 class ModelRunner:
@@ -99,6 +101,7 @@ class ModelRunner:
         self.stream.wait_stream(torch.cuda.current_stream(self.device))
         self.arena = Arena(self.device)
         self._kv_layers = sum(1 for need in model.cache_needs if need is not None and hasattr(need, "kv_heads"))
+        self.plans = model.batch_plans() if hasattr(model, "batch_plans") else []  # what the parts want of every batch
         self.link_norms = True  # see StepContext; set False before the first step to run every norm as a kernel of its own
         n_groups = len(manager.groups)
         # host mirror of every live request's block tables, one row per state slot
@@ -111,6 +114,7 @@ class ModelRunner:
         # captured steps by (rows of one token, tokens of prompt portions); recaptured wider when a request outgrows one
         self._graphs: dict[tuple[int, int], _StepGraph] = {}
         self._graph_uses = 0
+        self._graph_arena: Arena | None = None  # the newest (largest) arena of the captured steps
         self._pad_ready = False
         self._staged: torch.cuda.Event | None = None
         self.last_used_graph = False
@@ -233,12 +237,11 @@ class ModelRunner:
 
     def _step_eager(self, entries, rcs, starts, lens, n_want, device_tokens=None):
         n_tokens = sum(lens)
-        tc, td = count_tiles(lens)
         max_kv = max(s + n for s, n in zip(starts, lens))
         self.model.check_positions(max_kv - 1)
         width = max(1, -(-max_kv // self.page_size))
         n_patch = len(device_tokens[1]) if device_tokens else 0
-        layout = BatchLayout(n_tokens, len(entries), n_want, tc, td, len(self._tables), width, n_patch)
+        layout = BatchLayout(n_tokens, len(entries), n_want, len(self._tables), width, n_patch, plans=[(p, p.shape(lens)) for p in self.plans])
         if layout.total > self._host.numel():
             size = 1 << (layout.total - 1).bit_length()
             self._host = torch.zeros(size, dtype=torch.int32).pin_memory()
@@ -275,7 +278,9 @@ class ModelRunner:
 
     def _graph_shape(self, lens, n_want: int) -> tuple[int, int] | None:
         """(rows of one token, tokens of prompt portions) of the captured step that takes this batch, or None if it runs
-        eagerly: nothing wanted, more rows than the largest bucket, more or longer portions than a captured step holds."""
+        eagerly: nothing wanted, more rows than the largest bucket, more or longer portions than a captured step holds.  The
+        rows of a step that holds portions are padded to a multiple of ``MIXED_TOKEN_STEP``, up to 63 rows more than the
+        requests bring (the scheduler's token budget counts what they bring)."""
         if not n_want:
             return None
         singles = sum(1 for n in lens if n == 1)
@@ -373,26 +378,49 @@ class ModelRunner:
         g.used = self._graph_uses
         return g
 
+    def _arena_for(self, nbytes: int) -> Arena:
+        """The arena that a step captured now takes its intermediates from.  Captured steps replay one after another on
+        the runner's stream, so all of them share one arena as large as the largest of them needs; a step that needs more
+        than the arena has gets a new one, of the next power of two, which the steps captured later share.  Steps
+        captured earlier keep the arena they were captured with until they are dropped, so all arenas together are less
+        than twice the largest plus what dropped steps have not given back yet: the intermediates of one step, not of
+        ``MAX_GRAPHS``."""
+        have = self._graph_arena
+        if have is None or have.capacity < nbytes:
+            have = self._graph_arena = Arena(self.device, nbytes=1 << max(20, (nbytes - 1).bit_length()), fixed=True)
+        return have
+
+    @property
+    def graph_arena_bytes(self) -> int:
+        """Bytes of intermediates that the captured steps hold together (each shared arena counted once)."""
+        arenas = {id(g.arena): g.arena for g in self._graphs.values() if g.arena is not None}
+        if self._graph_arena is not None:
+            arenas[id(self._graph_arena)] = self._graph_arena
+        return sum(a.capacity for a in arenas.values())
+
     def _capture(self, shape: tuple[int, int], width: int) -> _StepGraph:
+        self._ensure_pad()
         g = _StepGraph(self, shape[0], shape[1], width)
         self._fill_graph(g, [], [], [], [])
-        ctx = g.context(self)
 
-        def run():
-            g.arena.reset()
+        def run(ctx):
+            ctx.arena.reset()
             resid, delta = self.model.forward_hidden(ctx, self.storage.views)
             logits = self.model.logits(ctx, resid, delta, ctx.want_rows)
             temp, top_p, uni, top_k = g.sample_options()
             ops.sample(logits, temp, uni, top_k=top_k, top_p=top_p, out=g.sampled)
             return logits
 
-        run()  # warm-up: loads the libraries and lets the arena grow to what a step needs
+        # a run outside the capture, in an arena that grows: it loads the libraries and measures what the step needs
+        probe = Arena(self.device)
+        run(g.context(self, probe))
         self.stream.synchronize()
-        g.arena.reset()  # one chunk from here on
-        g.arena.fixed = True
+        g.arena = self._arena_for(probe.high_water)
+        del probe
+        ctx = g.context(self, g.arena)
         graph = ops.Graph(self.stream)
         with graph:
-            g.logits = run()
+            g.logits = run(ctx)
         g.graph = graph
         self._graphs[shape] = g
         return g

@@ -10,10 +10,13 @@ A request's tokens are ``prompt + output``; ``computed`` of them are in the cach
 request brings its next tokens: exactly one when it is decoding, a portion when (part of) its prompt is
 still to be computed.  It samples in the step that consumes its last known token.
 
-Token budget (``max_step_tokens``): decoding requests come first with one token each (counted as
-``decode_rows_cost`` says: the engine rounds them up to the rows of a captured step, so that a step with its
-padding stays within the budget); what is left is given to unfinished prompts in admission order, at most
-``prefill_chunk`` tokens per request and step.
+Token budget (``max_step_tokens``): decoding requests come first with one token each.  The engine pads them to the
+rows of a captured step, and ``decode_rows_cost`` says to how many: where the padded rows fit the budget they are what
+is charged, so that prompts get what the padding leaves and a step of decode rows and its padding stays within the
+budget; where they do not fit, the rows are charged as what they are (the padding then goes beyond the budget rather
+than requests that would fit being left out).  What is left is given to unfinished prompts in admission order, at most
+``prefill_chunk`` tokens per request and step.  The budget bounds the tokens that requests bring; the engine may pad a
+step of prompt portions beside decode rows by up to 63 rows more to reach a captured shape.
 When the budget does not even cover the decoding requests, those that have waited longest since their
 last step go first (so that all of them advance in turn), and an eighth of the budget (at least one
 token) is kept for the oldest unfinished prompt, so that it advances too.
@@ -190,18 +193,20 @@ class Scheduler:
         work: list[Work] = []
         decoding = [r for r in self.running if r.seq_len - r.computed == 1]
         filling = [r for r in self.running if r.seq_len - r.computed > 1]
-        cost = self.decode_rows_cost
-        if budget is not None and cost(len(decoding)) + (1 if filling else 0) > budget:
+
+        def cost(n: int, room: int) -> int:
+            """What ``n`` rows of one token take of ``room`` tokens: with their padding if that fits, else as they are."""
+            padded = self.decode_rows_cost(n)
+            return padded if padded <= room else n
+
+        if budget is not None and len(decoding) + (1 if filling else 0) > budget:
             # not every decoding request fits: the longest-waiting first, and a share for the oldest unfinished prompt
             share = max(1, budget // 8) if filling and budget > 1 else 0
-            fit = len(decoding)
-            while fit and cost(fit) > budget - share:
-                fit -= 1
-            decoding = sorted(decoding, key=lambda r: r.served_at)[:fit]
+            decoding = sorted(decoding, key=lambda r: r.served_at)[: max(0, budget - share)]
         for r in decoding:
             work.append(Work(r, r.computed, 1))
         if budget is not None:
-            budget -= cost(len(decoding))
+            budget -= cost(len(decoding), budget - (1 if filling else 0))
         for r in filling:
             n = r.seq_len - r.computed
             if self.prefill_chunk is not None:

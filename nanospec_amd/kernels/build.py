@@ -124,8 +124,13 @@ def attn(head_dim: int, page_size: int) -> ctypes.CDLL:
     return load_library(attn_name(head_dim, page_size), ATTN_SOURCES, _attn_defines(head_dim, page_size))
 
 
-def build_all(attn_variants=((16, 4), (32, 8), (64, 16), (128, 16)), force: bool = True) -> None:
-    """Compile the core library and the attention library of each given (head size, page size)."""
-    compile_library("ns_core", CORE_SOURCES, force=force)
-    for hd, page in attn_variants:
-        compile_library(attn_name(hd, page), ATTN_SOURCES, _attn_defines(hd, page), force=force)
+def build_all(attn_variants=((16, 4), (32, 8), (64, 16), (128, 16)), force: bool = True, jobs: int | None = None) -> None:
+    """Compile the core library and the attention library of each given (head size, page size), ``jobs`` compilers at a
+    time (by default one per processor, at most eight)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    work = [("ns_core", CORE_SOURCES, [])] + [(attn_name(hd, page), ATTN_SOURCES, _attn_defines(hd, page)) for hd, page in attn_variants]
+    jobs = jobs or max(1, min(8, os.cpu_count() or 1))
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        for done in [pool.submit(compile_library, name, sources, defines, force) for name, sources, defines in work]:
+            done.result()

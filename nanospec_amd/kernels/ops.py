@@ -80,8 +80,8 @@ def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
 # ------------------------------------------------------------------------------------------------ elementwise
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[i] = table[ids[i]].  ``ids`` int32; the caller has checked 0 <= id < vocab."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+    """out[i] = table[ids[i]] (times ``scale``, in 32-bit, rounded once).  ``ids`` int32; the caller has checked 0 <= id < vocab."""
     _gpu(table, ids)
     _i32(ids, "ids")
     n, hidden = ids.numel(), table.shape[1]
@@ -89,8 +89,19 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = Non
         out = torch.empty((n, hidden), dtype=table.dtype, device=table.device)
     if not table.is_contiguous() or out.shape != (n, hidden) or out.dtype != table.dtype or not out.is_contiguous():
         raise KernelRefused("embed: table and out must be contiguous [*, hidden] of one dtype")
-    _check(build.core().ns_embed(_ptr(out), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), c_int(_dtype_code(table)), _stream()), "embed")
+    _check(build.core().ns_embed(_ptr(out), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), c_float(scale), c_int(_dtype_code(table)),
+                                 _stream()), "embed")
     return out
+
+
+def logit_transform(logits: torch.Tensor, scale: float = 1.0, softcap: float = 0.0) -> torch.Tensor:
+    """32-bit logits in place: times ``scale``; with ``softcap`` > 0 then softcap * tanh(logit / softcap)."""
+    _gpu(logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1 or softcap < 0:
+        raise KernelRefused("logit_transform takes float32 [rows, vocab] and a cap that is not negative")
+    _check(build.core().ns_logit_transform(_ptr(logits), c_int(logits.shape[0]), c_int(logits.shape[1]), c_int(logits.stride(0)),
+                                           c_float(scale), c_float(softcap), _stream()), "logit_transform")
+    return logits
 
 
 class PartialSums:
@@ -159,30 +170,46 @@ def rmsnorm(weight: torch.Tensor, eps: float, resid: torch.Tensor | None = None,
     return out
 
 
+def _check_pages(block_table, k_cache, v_cache, kv_heads: int, head_dim: int, dtype, what: str) -> int:
+    """What the kernels that write keys and values into pages assume of the pools and the block table.  -> page size.
+    (Positions and request indices inside the batch are the batch builder's: a kernel computes
+    ``block_table[token_req[t]][position // page]`` without asking whether the table is that wide.)"""
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelRefused(f"{what}: key pages are [pages, kv_heads, page, head_dim], value pages [pages, kv_heads, head_dim, page]")
+    page = k_cache.shape[2]
+    if (k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+            or k_cache.dtype != dtype or v_cache.dtype != dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused(f"{what}: cache pages do not fit heads, head size or dtype")
+    _i32(block_table, "block_table")
+    if block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelRefused(f"{what}: block_table is int32 [requests, pages] with unit stride along a row")
+    return page
+
+
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor, block_table: torch.Tensor,
                   inv_freq: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int, kv_heads: int,
-                  head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
+                  head_dim: int, rotary_dim: int, write_kv: bool = True, interleaved: bool = False, factor: float = 1.0) -> None:
     """Rotate q in place inside ``qkv`` [N, (heads + 2 kv_heads) * head_dim]; rotate k and write k and v of
     every token into the pages ``block_table[token_req[t], position // page]``.
-    k_cache [pages, kv_heads, page, head_dim]; v_cache [pages, kv_heads, head_dim, page]."""
+    k_cache [pages, kv_heads, page, head_dim]; v_cache [pages, kv_heads, head_dim, page].
+    ``interleaved``: pair j of the rotary part is channels (2j, 2j + 1) instead of (j, j + rotary_dim / 2); ``factor``
+    multiplies cosine and sine."""
     _gpu(qkv, positions, token_req, block_table, inv_freq, k_cache, v_cache)
     n = positions.numel()
     width = (heads + 2 * kv_heads) * head_dim
     if qkv.dim() != 2 or qkv.shape[0] != n or qkv.shape[1] != width or qkv.stride(1) != 1:
         raise KernelRefused(f"rope_kv_write: qkv must be [{n}, {width}]")
-    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
-    if token_req.numel() != n or block_table.dim() != 2:
-        raise KernelRefused("rope_kv_write: token_req is per token, block_table is [requests, pages]")
+    _i32(positions, "positions"), _i32(token_req, "token_req")
+    if token_req.numel() != n:
+        raise KernelRefused("rope_kv_write: token_req is per token")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2):
         raise KernelRefused("rope_kv_write: inv_freq must hold rotary_dim/2 float32 values")
-    page = k_cache.shape[2]
-    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
-            or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
-        raise KernelRefused("rope_kv_write: cache pages do not fit heads, head size or dtype")
+    page = _check_pages(block_table, k_cache, v_cache, kv_heads, head_dim, qkv.dtype, "rope_kv_write")
     _check(build.core().ns_rope_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
                                          c_int(block_table.stride(0)), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(n),
-                                         c_int(heads), c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(page),
-                                         c_int(1 if write_kv else 0), c_int(_dtype_code(qkv)), _stream()), "rope_kv_write")
+                                         c_int(heads), c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(1 if interleaved else 0),
+                                         c_float(factor), c_int(page), c_int(1 if write_kv else 0), c_int(_dtype_code(qkv)), _stream()),
+           "rope_kv_write")
 
 
 def silu_mul(gu: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -391,15 +418,17 @@ def linear_resid_norm(x: torch.Tensor, w: TiledWeight, resid: torch.Tensor, next
     return PreNormed(x_next, ssq, w.n, eps)
 
 
-def wide_plan(n: int, k: int, rows: int = SKINNY_MAX_ROWS) -> tuple[int, int]:
+def wide_plan(n: int, k: int, rows: int = SKINNY_MAX_ROWS, units: int | None = None) -> tuple[int, int]:
     """(ranges K is cut into, 16-row tiles per wave) of ``linear_wide``: two tiles per wave when there are rows enough
     (and at most 64 rows of x), then as many ranges as give every compute unit about one workgroup, with at least four k
     tiles of 128 per range (more, shorter ranges were measured slower once the kernel that joins them is counted: 37 against
-    31 us for the down-projection of the 8B shape at 64 rows with 10 and with 4 ranges)."""
+    31 us for the down-projection of the 8B shape at 64 rows with 10 and with 4 ranges).  ``units``: the GPU's compute
+    units (the current device's by default)."""
+    units = units or compute_units(torch.cuda.current_device())
     nt = 2 if n >= 8192 and rows <= SKINNY_MAX_ROWS else 1
     row_groups = -(-n // (64 * nt))
     k_tiles = -(-k // 128)
-    return max(1, min(16, k_tiles // 4, round(256 / row_groups))), nt
+    return max(1, min(16, k_tiles // 4, round(units / row_groups))), nt
 
 
 def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
@@ -439,13 +468,14 @@ def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, 
     return PartialSums(workspace, ksplit, m, w.n, x.dtype) if defer else out
 
 
-def rows_plan(n: int, k: int, rows: int, gated: bool = False) -> tuple[int, int]:
+def rows_plan(n: int, k: int, rows: int, gated: bool = False, units: int | None = None) -> tuple[int, int]:
     """(ranges K is cut into, 16-row tiles per wave) of ``linear_rows``: the most tiles per wave, then ranges of K until
     the workgroups fill the GPU, with at least eight k tiles of 128 per range."""
+    units = units or compute_units(torch.cuda.current_device())
     nt = 2 if gated else 4
     groups = -(-n // (64 * nt)) * -(-rows // 128)
     k_tiles = -(-k // 128)
-    return max(1, min(16, k_tiles // 8, 256 // groups)), nt
+    return max(1, min(16, k_tiles // 8, units // groups)), nt
 
 
 def linear_rows(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
@@ -480,16 +510,18 @@ def linear_rows(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, 
     return out
 
 
-def qkv_rope_row_order(heads: int, kv_heads: int, head_dim: int, rotary_dim: int) -> torch.Tensor:
+def qkv_rope_row_order(heads: int, kv_heads: int, head_dim: int, rotary_dim: int, interleaved: bool = False) -> torch.Tensor:
     """The row order of a stacked [q; k; v] matrix for ``linear_qkv_rope``: per head 16-row tiles; in the rotary part of a
-    q or k head a tile holds 8 channels j and their partners j + rotary_dim/2, elsewhere 16 consecutive channels."""
+    q or k head a tile holds the first channels of 8 rotary pairs and then their second channels (pair j is channels j and
+    j + rotary_dim/2, or 2j and 2j + 1 with ``interleaved``), elsewhere 16 consecutive channels."""
     order = []
     half = rotary_dim // 2
+    first, second = ((lambda j: 2 * j), (lambda j: 2 * j + 1)) if interleaved else ((lambda j: j), (lambda j: j + half))
     for g in range(heads + 2 * kv_heads):
         base = g * head_dim
         rot = rotary_dim if g < heads + kv_heads else 0
         for jt in range(rot // 16):
-            order += [base + jt * 8 + e for e in range(8)] + [base + half + jt * 8 + e for e in range(8)]
+            order += [base + first(jt * 8 + e) for e in range(8)] + [base + second(jt * 8 + e) for e in range(8)]
         for d0 in range(rot, head_dim, 16):
             order += [base + d0 + e for e in range(16)]
     return torch.tensor(order, dtype=torch.int64)
@@ -501,10 +533,10 @@ def qkv_rope_takes(x: torch.Tensor, head_dim: int, rotary_dim: int) -> bool:
 
 def linear_qkv_rope(x: "torch.Tensor | PreNormed", w: TiledWeight, q_out: torch.Tensor, positions, token_req, block_table, inv_freq,
                     k_cache, v_cache, heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True,
-                    waves: int = 0) -> None:
+                    waves: int = 0, interleaved: bool = False, factor: float = 1.0) -> None:
     """The stacked q/k/v product of at most 16 tokens with rotation and cache write fused into its epilogue: q goes rotated
     into ``q_out`` [M, >= heads * head_dim], k rotated into its K page slot, v into the transposed V page.  ``w`` is the
-    stacked matrix tiled in ``qkv_rope_row_order``.  ``x`` may be a ``PreNormed``."""
+    stacked matrix tiled in ``qkv_rope_row_order`` (of the same ``interleaved``).  ``x`` may be a ``PreNormed``."""
     pre = x if isinstance(x, PreNormed) else None
     if pre is not None:
         x = pre.x
@@ -516,11 +548,8 @@ def linear_qkv_rope(x: "torch.Tensor | PreNormed", w: TiledWeight, q_out: torch.
         raise KernelRefused("linear_qkv_rope: the weight does not hold heads + 2 kv_heads heads")
     if q_out.dtype != torch.bfloat16 or q_out.shape[0] != m or q_out.shape[1] < heads * head_dim or q_out.stride(1) != 1:
         raise KernelRefused("linear_qkv_rope: q_out must be bfloat16 [rows, >= heads * head_dim]")
-    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
-    page = k_cache.shape[2]
-    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
-            or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
-        raise KernelRefused("linear_qkv_rope: cache pages do not fit heads, head size or dtype")
+    _i32(positions, "positions"), _i32(token_req, "token_req")
+    page = _check_pages(block_table, k_cache, v_cache, kv_heads, head_dim, torch.bfloat16, "linear_qkv_rope")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2) or positions.numel() != m or token_req.numel() != m:
         raise KernelRefused("linear_qkv_rope: positions, token_req are per row; inv_freq holds rotary_dim / 2 float32 values")
     if waves == 0:
@@ -528,15 +557,17 @@ def linear_qkv_rope(x: "torch.Tensor | PreNormed", w: TiledWeight, q_out: torch.
     _check(build.core().ns_gemm_qkv_rope_bf16(_ptr(q_out), _ptr(x), _ptr(w.data), c_int(m), c_int(w.k), c_int(x.stride(0)),
                                               c_int(q_out.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
                                               c_int(block_table.stride(0)), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(heads),
-                                              c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(page),
+                                              c_int(kv_heads), c_int(head_dim), c_int(rotary_dim), c_int(1 if interleaved else 0),
+                                              c_float(factor), c_int(page),
                                               c_int(1 if write_kv else 0), c_int(waves), *_prenorm_args(pre, m, "linear_qkv_rope"),
                                               _stream()), "linear_qkv_rope")
 
 
 def rope_kv_from_partial(p: PartialSums, q_out: torch.Tensor, positions, token_req, block_table, inv_freq, k_cache, v_cache,
-                         heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
+                         heads: int, kv_heads: int, head_dim: int, rotary_dim: int, write_kv: bool = True, interleaved: bool = False,
+                         factor: float = 1.0) -> None:
     """Rotation and cache write for a stacked q/k/v product whose K ranges are not added up yet (``linear_wide(...,
-    defer=True)`` from a weight tiled in ``qkv_rope_row_order``): one pass adds the ranges, rotates, and writes q into
+    defer=True)`` from a weight tiled in ``qkv_rope_row_order`` of the same ``interleaved``): one pass adds the ranges, rotates, and writes q into
     ``q_out`` [rows, >= heads * head_dim], k into its K page slot and v into the transposed V page."""
     _gpu(p.ws, q_out, positions, token_req, block_table, inv_freq, k_cache, v_cache)
     m = p.rows
@@ -544,11 +575,8 @@ def rope_kv_from_partial(p: PartialSums, q_out: torch.Tensor, positions, token_r
         raise KernelRefused("rope_kv_from_partial takes a bfloat16 product of heads + 2 kv_heads heads, head and rotary sizes multiples of 16")
     if q_out.dtype != torch.bfloat16 or q_out.shape[0] != m or q_out.shape[1] < heads * head_dim or q_out.stride(1) != 1:
         raise KernelRefused("rope_kv_from_partial: q_out must be bfloat16 [rows, >= heads * head_dim]")
-    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
-    page = k_cache.shape[2]
-    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
-            or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
-        raise KernelRefused("rope_kv_from_partial: cache pages do not fit heads, head size or dtype")
+    _i32(positions, "positions"), _i32(token_req, "token_req")
+    page = _check_pages(block_table, k_cache, v_cache, kv_heads, head_dim, torch.bfloat16, "rope_kv_from_partial")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rotary_dim // 2) or positions.numel() != m or token_req.numel() != m:
         raise KernelRefused("rope_kv_from_partial: positions, token_req are per row; inv_freq holds rotary_dim / 2 float32 values")
     if p.ws.dtype != torch.float32 or p.ws.numel() < p.ksplit * m * p.n:
@@ -556,7 +584,8 @@ def rope_kv_from_partial(p: PartialSums, q_out: torch.Tensor, positions, token_r
     _check(build.core().ns_rope_kv_partial(_ptr(q_out), c_int(q_out.stride(0)), _ptr(p.ws), c_int(p.ksplit), c_int(m), c_int(p.n),
                                            _ptr(positions), _ptr(token_req), _ptr(block_table), c_int(block_table.stride(0)),
                                            _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), c_int(heads), c_int(kv_heads), c_int(head_dim),
-                                           c_int(rotary_dim), c_int(page), c_int(1 if write_kv else 0), _stream()), "rope_kv_from_partial")
+                                           c_int(rotary_dim), c_int(1 if interleaved else 0), c_float(factor), c_int(page),
+                                           c_int(1 if write_kv else 0), _stream()), "rope_kv_from_partial")
 
 
 # ------------------------------------------------------------------------------------------------ attention

@@ -13,6 +13,7 @@ import torch
 from .config import load_config
 from .parts import DecoderModel
 from .weights import DictSource, SafetensorsSource, random_tensors
+from .weights.random_init import draw
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
 
@@ -74,7 +75,6 @@ def random_model(config, seed: int = 0, device="cuda", dtype=torch.bfloat16, on_
 
         def get(self, name):
             shape, role = self.wanted[name]
-            t = torch.empty(shape, dtype=dtype, device=device).normal_(0.0, 0.02, generator=self.gen)
-            return t + 1.0 if role == "norm" else t
+            return draw(shape, role, self.gen, dtype, dtype)
 
     return net.load(_Lazy(net.wanted()), dtype, device, layouts)

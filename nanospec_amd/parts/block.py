@@ -45,6 +45,9 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def batch_plans(self) -> list:
+        return [plan for p in self.parts for plan in getattr(p, "batch_plans", list)()]
+
     def max_positions(self) -> int | None:
         """The positions the block's parts can encode; None if nothing bounds them."""
         limits = [p.max_positions() for p in self.parts if hasattr(p, "max_positions")]

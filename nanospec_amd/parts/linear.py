@@ -30,14 +30,32 @@ STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the sha
 WIDE_HEAD_ROWS = 12  # above this many rows a wide 32-bit product (the head) is faster through the 17-to-64-row kernel
 WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
 #                    32-bit results, which the library does not give); wider products go to the library
-PLAIN_SLICE_K = 8192  # such a copy of a matrix on its way into the residual stream is made and used in slices of the inner
-#                       size no longer than this (the scratch stays small, and no product runs longer over K than the ones
-#                       that were measured)
+LIBRARY_MAX_K = 14336  # the longest inner size over which the library's product has run here, kernel by kernel and inside
+#                        captured steps, with every replay checked.  ``library_product`` refuses a longer one: such a product is cut
+#                        into slices of its inner size in steps that are launched kernel by kernel, and runs through the
+#                        hand-written kernels in captured steps, whichever layouts are kept.
+PLAIN_SLICE_K = 8192  # the slices of a product on its way into the residual stream that is cut along its inner size are no
+#                       longer than this (where only the re-laid copy is kept the scratch copy is then a slice, not the
+#                       matrix, and products are cut from this size on already)
 UNTILE_MIN_ROWS = 768  # where only the re-laid copy is kept: from this many rows on the products whose callers allow it
 #                        (``plain_copy``: q/k/v, o, gate/up, down) first write their matrices out in plain rows (scratch) and go to
 #                        the library; the copy costs what 300 rows of the product cost, and the library is 1.6 to 2 times as
 #                        fast as the many-row kernel (measured at the 70B shape).  Callers allow it in steps that are launched
 #                        kernel by kernel only: the scratch is as large as the matrix, and every captured step keeps its own.
+
+
+def library_product(x: torch.Tensor, w_t: torch.Tensor, out: torch.Tensor | None = None, into: torch.Tensor | None = None) -> torch.Tensor:
+    """The one door to the platform's GEMM library: x @ w_t (``w_t`` [in, out], usually the transposed view of a matrix
+    in plain rows).  ``into``: the product is added to this tensor in place, summed in 32-bit and rounded once; a 32-bit
+    ``into`` beside bfloat16 operands keeps the sum in 32-bit.  An inner size beyond ``LIBRARY_MAX_K`` is refused: the
+    library chooses other kernels for it, none of which has run here."""
+    if x.shape[1] > LIBRARY_MAX_K:
+        raise ops.KernelRefused(f"a library product over an inner size of {x.shape[1]} (more than {LIBRARY_MAX_K}) must be cut into slices")
+    if into is not None:
+        if into.dtype == torch.float32 and x.dtype != torch.float32:
+            return torch.addmm(into, x, w_t, out_dtype=torch.float32, out=into)
+        return into.addmm_(x, w_t)
+    return torch.matmul(x, w_t) if out is None else torch.matmul(x, w_t, out=out)
 
 
 class IntoResidual:
@@ -68,7 +86,8 @@ class LinearWeight:
         self.n, self.k = w.shape
         self.dtype = w.dtype
         fast = w.dtype == torch.bfloat16 and self.k % 8 == 0
-        self.tiled = ops.TiledWeight(w) if (fast and tiled) else None
+        # (an inner size that the library does not take in one piece needs the hand-written kernels for many rows too)
+        self.tiled = ops.TiledWeight(w) if (fast and (tiled or self.k > LIBRARY_MAX_K)) else None
         self.plain = w if (keep_plain or self.tiled is None) else None
         self._plain_t = self.plain.t() if self.plain is not None else None  # the library product's operand, made once
 
@@ -101,29 +120,32 @@ class LinearWeight:
         # rounded once, so the norm after it reads one tensor instead of two and writes one instead of two
         library = (m > ops.SKINNY_MAX_ROWS and x.dtype == torch.bfloat16 and r.dtype == torch.bfloat16 and r.shape == (m, self.n)
                    and r.is_contiguous())
-        plain_t = self._plain_t
-        if (library and plain_t is None and plain_copy and self.tiled is not None and m >= UNTILE_MIN_ROWS
-                and ops.tiled_takes(x[:1], self.k)):  # only the re-laid copy is kept, many rows
-            if self.k > PLAIN_SLICE_K:
-                # a long inner size in slices: the stream in 32-bit takes every slice's product as the library adds it
-                # (32-bit sums, 32-bit addend and result) and is rounded once at the end, as one product would be
-                slices = -(-self.k // PLAIN_SLICE_K)
-                width = -(-self.k // (128 * slices)) * 128
-                acc = take((m, self.n), torch.float32)
-                acc.copy_(r)
-                plain = take((self.n, width), self.dtype)
-                for k0 in range(0, self.k, width):
-                    k1 = min(self.k, k0 + width)
-                    piece = ops.untile(self.tiled, plain[:, : k1 - k0], k0, k1)
-                    torch.addmm(acc, x[:, k0:k1], piece.t(), out_dtype=torch.float32, out=acc)
-                r.copy_(acc)
+        have_plain = self._plain_t is not None
+        # only the re-laid copy is kept: many rows of a step that is launched kernel by kernel may copy it into plain rows
+        can_copy = (not have_plain and plain_copy and self.tiled is not None and m >= UNTILE_MIN_ROWS and ops.tiled_takes(x[:1], self.k))
+        if library and (have_plain or can_copy):
+            if self.k > (LIBRARY_MAX_K if have_plain else PLAIN_SLICE_K):
+                if plain_copy:
+                    # a long inner size in slices: the stream in 32-bit takes every slice's product as the library adds it
+                    # (32-bit sums, 32-bit addend and result) and is rounded once at the end, as one product would be
+                    slices = -(-self.k // PLAIN_SLICE_K)
+                    width = -(-self.k // (128 * slices)) * 128
+                    acc = take((m, self.n), torch.float32)
+                    acc.copy_(r)
+                    scratch = None if have_plain else take((self.n, width), self.dtype)
+                    for k0 in range(0, self.k, width):
+                        k1 = min(self.k, k0 + width)
+                        piece = self.plain[:, k0:k1] if have_plain else ops.untile(self.tiled, scratch[:, : k1 - k0], k0, k1)
+                        library_product(x[:, k0:k1], piece.t(), into=acc)
+                    r.copy_(acc)
+                    return ops.Added()
+                # (a captured step: the hand-written kernels below)
+            else:
+                plain_t = self._plain_t if have_plain else ops.untile(self.tiled, take((self.n, self.k), self.dtype)).t()
+                library_product(x, plain_t, into=r)
                 return ops.Added()
-            plain_t = ops.untile(self.tiled, take((self.n, self.k), self.dtype)).t()
-        if library and plain_t is not None:
-            r.addmm_(x, plain_t)
-            return ops.Added()
         out = link.x_next if link.x_next is not None else take((m, self.n), x.dtype)
-        return self(x, out=out, arena=arena)
+        return self(x, out=out, arena=arena, plain_copy=plain_copy)
 
     def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None, plain_copy: bool = False) -> torch.Tensor:
         """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated.
@@ -151,15 +173,15 @@ class LinearWeight:
             ksplit, nt = ops.wide_plan(self.n, self.k, m)
             ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
             return ops.linear_wide(x, self.tiled, out=out, out_f32=out_f32, workspace=ws, ksplit=ksplit, nt=nt)
-        if self.plain is not None and (not out_f32 or self.tiled is None):
+        if self.plain is not None and (not out_f32 or self.tiled is None) and (self.k <= LIBRARY_MAX_K or self.tiled is None):
             if out_f32:
                 return ops.linear_generic(x, self.plain, out=out, out_f32=True)
-            return torch.matmul(x, self._plain_t) if out is None else torch.matmul(x, self._plain_t, out=out)
+            return library_product(x, self._plain_t, out=out)
         if out is None:
             out = torch.empty((m, self.n), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
-        if m >= UNTILE_MIN_ROWS and not out_f32 and plain_copy and self.k <= PLAIN_SLICE_K:  # only the tiled layout is kept, many rows: a plain copy for this one product
+        if self.plain is None and m >= UNTILE_MIN_ROWS and not out_f32 and plain_copy and self.k <= PLAIN_SLICE_K:  # only the tiled layout is kept, many rows: a plain copy for this one product
             plain = arena.take((self.n, self.k), self.dtype) if arena is not None else torch.empty((self.n, self.k), dtype=self.dtype, device=x.device)
-            return torch.matmul(x, ops.untile(self.tiled, plain).t(), out=out)
+            return library_product(x, ops.untile(self.tiled, plain).t(), out=out)
         if m > ops.WIDE_TALL_ROWS:  # ... fewer: blocks of 128 rows through the hand-written kernel
             ksplit, nt = ops.rows_plan(self.n, self.k, m)
             ws = arena.take((ksplit * m * self.n,), torch.float32) if (arena is not None and ksplit > 1) else None
@@ -198,19 +220,21 @@ class GatedWeights:
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
-        if fast and self.stacked is None and m >= UNTILE_MIN_ROWS and not ctx.captured:
+        # (an inner size that the library does not take in one piece: the hand-written kernels at every number of rows)
+        stacked = self.stacked if (self.k <= LIBRARY_MAX_K or not fast) else None
+        if fast and stacked is None and self.k <= LIBRARY_MAX_K and m >= UNTILE_MIN_ROWS and not ctx.captured:
             # only the tiled layout is kept, many rows: both matrices in plain rows into scratch, then as with both layouts
             # (not in a captured step: every captured shape would hold a scratch of its own as large as the two matrices)
             stacked = ctx.arena.take((2 * self.inter, self.k), x.dtype)
             ops.untile(self.tiled[0], stacked[: self.inter])
             ops.untile(self.tiled[1], stacked[self.inter :])
             gu = ctx.arena.take((m, 2 * self.inter), x.dtype)
-            torch.matmul(x, stacked.t(), out=gu)
+            library_product(x, stacked.t(), out=gu)
             return ops.silu_mul(gu, out=out)
-        if fast and self.stacked is None and m > ops.WIDE_TALL_ROWS:
+        if fast and stacked is None and m > ops.WIDE_TALL_ROWS:
             # only the tiled layout is kept: blocks of 128 rows through the hand-written kernel, activation in the same pass
             return ops.linear_rows(x, self.tiled[0], w2=self.tiled[1], out=out, ksplit=1, nt=2)
-        if fast and (m <= ops.SKINNY_MAX_ROWS or self.stacked is None):
+        if fast and (m <= ops.SKINNY_MAX_ROWS or stacked is None):
             # 17 to 64 rows: the second hand-written kernel, one range of K, so that the activation is applied in the same
             # pass (measured ahead of the library's product plus the activation kernel)
             for s in range(0, m, ops.SKINNY_MAX_ROWS):
@@ -221,5 +245,5 @@ class GatedWeights:
         if self.dtype == torch.float32 or self.k % 8:
             ops.linear_generic(x, self.stacked, out=gu)
         else:
-            torch.matmul(x, self._stacked_t, out=gu)
+            library_product(x, self._stacked_t, out=gu)
         return ops.silu_mul(gu, out=out)

@@ -46,6 +46,14 @@ class DecoderModel:
     def graph_safe(self) -> bool:
         return all(layer.graph_safe for layer in self.layers)
 
+    def batch_plans(self) -> list:
+        """The batch plans of all layers' parts, one per key (``engine.context``)."""
+        plans = {}
+        for layer in self.layers:
+            for plan in getattr(layer, "batch_plans", list)():
+                plans.setdefault(plan.key, plan)
+        return list(plans.values())
+
     def wanted(self) -> dict:
         return wanted_tensors(self.spec, self.layers)
 
@@ -112,7 +120,7 @@ class DecoderModel:
         n = ctx.n_tokens
         resid = ctx.arena.take((n, self.spec.hidden), self.dtype)
         delta = ctx.arena.take((n, self.spec.hidden), self.dtype)
-        ops.embed(self.embed, ctx.token_ids, out=resid)
+        ops.embed(self.embed, ctx.token_ids, out=resid, scale=self.spec.embed_scale)
         pending = None
         order = self.spec.run_order
         # buffers for what one block hands to the next (see PreNormBlock.forward)
@@ -139,4 +147,7 @@ class DecoderModel:
         (reference: model/llama.py:284-286, engine/engine.py:382)."""
         n = rows.numel()
         h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
-        return self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True, arena=ctx.arena)
+        out = self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True, arena=ctx.arena)
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap:
+            ops.logit_transform(out, self.spec.logit_scale, self.spec.logit_softcap)
+        return out

@@ -7,8 +7,9 @@ then built wherever a spec of that kind appears in a ``ModelSpec``.
 What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are [tokens, width]):
 
   every part   __init__(spec, prefix)             prefix: tensor-name prefix of its weights
-               wanted() -> {name: (shape, role)}   tensors it reads from the checkpoint; role is one of
-                                                  "linear" | "embedding" | "norm" (used by random init)
+               wanted() -> {name: (shape, role)}   tensors it reads from the checkpoint; role says how random weights
+                                                  are drawn: "linear" | "embedding" | "norm" | "zeros" | "ones", or a
+                                                  function (shape, generator) -> tensor (weights/random_init.py)
                load(get, dtype, device)           get(name) returns the stored tensor (CPU)
                graph_safe: bool                   True if forward only launches kernels on the current
                                                   stream into buffers taken from ctx.arena
@@ -23,6 +24,11 @@ What each role must offer (``ctx`` is the engine's ``StepContext``, tensors are 
                cache_need(); forward(ctx, resid, delta, cache, owns_cache, delta_out) -> None
                                                   resid is updated in place; the not yet added output of
                                                   the block's last part is left in delta_out
+
+Rows of a step may be padding (captured steps have fixed shapes): their inputs are arbitrary bits, NaNs included, and their
+outputs are never read.  A part keeps rows independent of each other (as every product, norm and per-token mixer does), or
+tells padding rows on the device by ``ctx.state_slots[ctx.token_req[row]] == ctx.pad_slot`` (``pad_slot`` is None in steps
+without padding).
 
 Optional:
   mixer, block max_positions() -> int | None      the positions it can encode (the engine refuses requests beyond the

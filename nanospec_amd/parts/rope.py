@@ -1,9 +1,13 @@
 """Rotary position encoding: the inverse frequencies, with the llama3 scaling of long wavelengths.
 
-Only the frequencies live here; the rotation itself is fused into the kernel that writes keys and
-values to the cache (``kernels.ops.rope_kv_write``), which forms angle = position * inv_freq and its
-cosine and sine in 32-bit.  Reference: model/llama.py:98-118 (frequencies), :133-136 (angles),
-:150-158 (pairing of element j with j + d/2).
+Only the frequencies and the form of the rotation live here (which elements make a pair, a factor on cosine and
+sine); the rotation itself is fused into the kernels that write keys and values to the cache (``kernels.ops.rope_kv_write``
+and the q/k/v products' epilogues, all through the one device function of ``csrc/rope.h``), which form
+angle = position * inv_freq and its cosine and sine in 32-bit.  Reference: model/llama.py:98-118 (frequencies),
+:133-136 (angles), :150-158 (pairing of element j with j + d/2).
+
+A position encoding of another kind that the attention part can apply is an object with ``inv_freq`` (float32 on the
+device, rotary_dim / 2 values), ``rotary_dim``, ``max_positions`` and optionally ``interleaved`` and ``factor``.
 """
 
 from __future__ import annotations
@@ -39,6 +43,7 @@ class Rope:
         self.spec = spec
         self.rotary_dim = spec.rotary_dim
         self.max_positions = spec.max_positions
+        self.interleaved, self.factor = bool(spec.interleaved), float(spec.cos_sin_factor)
         self.inv_freq: torch.Tensor | None = None
 
     def wanted(self) -> dict:
@@ -54,6 +59,7 @@ class NoPosition:
     graph_safe = True
     rotary_dim = 0
     max_positions = None
+    interleaved, factor = False, 1.0
 
     def __init__(self, spec, prefix: str = "") -> None:
         self.inv_freq = None

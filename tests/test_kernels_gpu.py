@@ -195,9 +195,27 @@ def scattered_tables(lens, page, pages, seed=0):
     return table
 
 
+FORMS = [(False, 1.0), (True, 0.75)]  # (pairs of channels 2j and 2j + 1 instead of j and j + d/2, a factor on cosine and sine)
+
+
+def plain_rotation(x, cos, sin, interleaved=False, factor=1.0):
+    """The rotation of x [T, heads, d] in the given form.  The half-split form is the plain implementation's; the
+    interleaved form turns channels 2j and 2j + 1 by the same angle j, written out here pair by pair."""
+    if not interleaved:
+        return pl.rotate(x, cos * factor, sin * factor)
+    half = x.shape[-1] // 2
+    c, s = (cos[:, None, :half] * factor), (sin[:, None, :half] * factor)
+    a, b = x.float()[..., 0::2], x.float()[..., 1::2]
+    out = torch.empty_like(x, dtype=torch.float32)
+    out[..., 0::2] = a * c - b * s
+    out[..., 1::2] = b * c + a * s
+    return out.to(x.dtype)
+
+
+@pytest.mark.parametrize("form", FORMS, ids=["halves", "interleaved"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rot", [24, 16, 0])
-def test_rope_kv_write(dtype, rot):
+def test_rope_kv_write(dtype, rot, form):
     """q rotated in place, k rotated into its page slot, v into the transposed page; against the plain rotation."""
     ops = _ops()
     torch.manual_seed(1)
@@ -211,14 +229,14 @@ def test_rope_kv_write(dtype, rot):
     before = qkv.clone().cpu()
     k, v = make_cache(16, page, kvh, hd, dtype)
     inv = pl.inverse_frequencies(rot, 10000.0, None) if rot else torch.zeros(1)
-    ops.rope_kv_write(qkv, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot)
+    ops.rope_kv_write(qkv, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot, interleaved=form[0], factor=form[1])
     q0 = before[:, : heads * hd].view(n, heads, hd)
     k0 = before[:, heads * hd : (heads + kvh) * hd].view(n, kvh, hd)
     v0 = before[:, (heads + kvh) * hd :].view(n, kvh, hd)
     if rot:
         cos, sin = pl.rotation_tables(positions.cpu(), inv)
-        q_ref = torch.cat([pl.rotate(q0[..., :rot], cos, sin), q0[..., rot:]], -1)
-        k_ref = torch.cat([pl.rotate(k0[..., :rot], cos, sin), k0[..., rot:]], -1)
+        q_ref = torch.cat([plain_rotation(q0[..., :rot], cos, sin, *form), q0[..., rot:]], -1)
+        k_ref = torch.cat([plain_rotation(k0[..., :rot], cos, sin, *form), k0[..., rot:]], -1)
     else:
         q_ref, k_ref = q0, k0
     tol = _tol(dtype)
@@ -231,8 +249,9 @@ def test_rope_kv_write(dtype, rot):
         assert torch.equal(v[pg, :, :, off].cpu(), v0[t])
 
 
+@pytest.mark.parametrize("form", FORMS, ids=["halves", "interleaved"])
 @pytest.mark.parametrize("heads,kvh,hd,rot,page", [(6, 3, 32, 32, 4), (4, 1, 48, 16, 8), (8, 2, 128, 128, 16), (2, 2, 16, 0, 4)])
-def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, page):
+def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, page, form):
     """One kernel for x @ [Wq; Wk; Wv]^T, the rotation of q and k and the write of k and v into their pages, against the
     plain product followed by the plain rotation."""
     ops = _ops()
@@ -245,19 +264,20 @@ def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, pa
     token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
     w = (torch.randn((heads + 2 * kvh) * hd, hidden) * 0.3).to(torch.bfloat16)
     x = torch.randn(n, hidden).to(torch.bfloat16)
-    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot))
+    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot, form[0]))
     q_out = torch.zeros(n, (heads + 2 * kvh) * hd, dtype=torch.bfloat16, device=DEV)
     k, v = make_cache(16, page, kvh, hd, torch.bfloat16)
     inv = pl.inverse_frequencies(rot, 10000.0, None) if rot else torch.zeros(1)
-    ops.linear_qkv_rope(x.to(DEV), wt, q_out, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot)
+    ops.linear_qkv_rope(x.to(DEV), wt, q_out, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot, interleaved=form[0],
+                        factor=form[1])
     full = x.float() @ w.float().T  # 32-bit sums: the kernel rotates before it rounds
     q0 = full[:, : heads * hd].view(n, heads, hd)
     k0 = full[:, heads * hd : (heads + kvh) * hd].view(n, kvh, hd)
     v0 = full[:, (heads + kvh) * hd :].view(n, kvh, hd)
     if rot:
         cos, sin = pl.rotation_tables(positions.cpu(), inv)
-        q0 = torch.cat([pl.rotate(q0[..., :rot], cos, sin), q0[..., rot:]], -1)
-        k0 = torch.cat([pl.rotate(k0[..., :rot], cos, sin), k0[..., rot:]], -1)
+        q0 = torch.cat([plain_rotation(q0[..., :rot], cos, sin, *form), q0[..., rot:]], -1)
+        k0 = torch.cat([plain_rotation(k0[..., :rot], cos, sin, *form), k0[..., rot:]], -1)
     assert ulps_of_row_max(q_out[:, : heads * hd].cpu(), q0.reshape(n, -1)).max() <= 1.0
     for t in range(n):
         b, p = int(token_req[t]), int(positions[t])
@@ -266,10 +286,11 @@ def test_qkv_product_with_fused_rotation_and_cache_write(heads, kvh, hd, rot, pa
         assert ulps_of_row_max(v[pg, :, :, off].cpu().reshape(1, -1), v0[t].reshape(1, -1)).max() <= 1.0
 
 
+@pytest.mark.parametrize("form", FORMS, ids=["halves", "interleaved"])
 @pytest.mark.parametrize("rows", [17, 40, 64, 100, 128])
 @pytest.mark.parametrize("heads,kvh,hd,rot,page,hidden,ksplit", [(6, 3, 32, 32, 4, 384, 3), (4, 1, 48, 16, 8, 520, 2), (8, 2, 128, 128, 16, 1024, 4),
                                                                  (2, 2, 16, 0, 4, 256, 2)])
-def test_qkv_product_in_ranges_joined_by_the_rotation_kernel(rows, heads, kvh, hd, rot, page, hidden, ksplit):
+def test_qkv_product_in_ranges_joined_by_the_rotation_kernel(rows, heads, kvh, hd, rot, page, hidden, ksplit, form):
     """17 to 128 rows: the stacked product with K cut into ranges from the matrix tiled in the few-row kernel's row order,
     and one kernel that adds the ranges, rotates q and k and writes k and v into their pages; against the plain product
     followed by the plain rotation.  Requests of several tokens and of one, pages scattered."""
@@ -284,21 +305,22 @@ def test_qkv_product_in_ranges_joined_by_the_rotation_kernel(rows, heads, kvh, h
     token_req = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
     w = (torch.randn((heads + 2 * kvh) * hd, hidden) * 0.3).to(torch.bfloat16)
     x = torch.randn(n, hidden).to(torch.bfloat16)
-    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot))
+    wt = ops.TiledWeight(w.to(DEV), ops.qkv_rope_row_order(heads, kvh, hd, rot, form[0]))
     q_out = torch.zeros(n, (heads + 2 * kvh) * hd, dtype=torch.bfloat16, device=DEV)
     k, v = make_cache(64, page, kvh, hd, torch.bfloat16)
     inv = pl.inverse_frequencies(rot, 10000.0, None) if rot else torch.zeros(1)
     part = ops.linear_wide(x.to(DEV), wt, ksplit=ksplit, nt=1, defer=True)
     assert isinstance(part, ops.PartialSums) and part.ksplit == ksplit
-    ops.rope_kv_from_partial(part, q_out, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot)
+    ops.rope_kv_from_partial(part, q_out, positions, token_req, table, inv.to(DEV), k, v, heads, kvh, hd, rot, interleaved=form[0],
+                             factor=form[1])
     full = x.float() @ w.float().T  # 32-bit sums: the kernel rotates before it rounds
     q0 = full[:, : heads * hd].view(n, heads, hd)
     k0 = full[:, heads * hd : (heads + kvh) * hd].view(n, kvh, hd)
     v0 = full[:, (heads + kvh) * hd :].view(n, kvh, hd)
     if rot:
         cos, sin = pl.rotation_tables(positions.cpu(), inv)
-        q0 = torch.cat([pl.rotate(q0[..., :rot], cos, sin), q0[..., rot:]], -1)
-        k0 = torch.cat([pl.rotate(k0[..., :rot], cos, sin), k0[..., rot:]], -1)
+        q0 = torch.cat([plain_rotation(q0[..., :rot], cos, sin, *form), q0[..., rot:]], -1)
+        k0 = torch.cat([plain_rotation(k0[..., :rot], cos, sin, *form), k0[..., rot:]], -1)
     assert ulps_of_row_max(q_out[:, : heads * hd].cpu(), q0.reshape(n, -1)).max() <= 1.0
     assert torch.count_nonzero(q_out[:, heads * hd :]) == 0  # only q goes to the attention input
     for t in range(n):

@@ -35,11 +35,11 @@ def make_ctx(lens, starts, tables, page, dtype, want=()):
     import numpy as np
 
     from nanospec_amd.engine.arena import Arena
-    from nanospec_amd.engine.context import BatchLayout, StepContext, count_tiles, fill_batch
+    from nanospec_amd.engine.context import BatchLayout, StepContext, fill_batch
+    from nanospec_amd.parts.attention import TILES
 
-    tc, td = count_tiles(lens)
     width = max(len(t) for t in tables)
-    layout = BatchLayout(sum(lens), len(lens), len(want), tc, td, 1, width)
+    layout = BatchLayout(sum(lens), len(lens), len(want), 1, width, plans=[(TILES, TILES.shape(lens))])
     host = np.zeros(layout.total, dtype=np.int32)
     table = np.full((len(lens), width), -1, dtype=np.int32)
     for b, t in enumerate(tables):
@@ -882,3 +882,170 @@ def test_an_architecture_registered_from_outside_generates(tmp_path):
     torch.testing.assert_close(out[0], plain(prompts[2][:20])[-1], rtol=1e-4, atol=1e-4)
     out = rep.step([{"id": "a", "tokens": prompts[2][20:], "want": [12]}, {"id": "b", "tokens": prompts[1][2:], "want": [16]}], ["a", "b"])
     torch.testing.assert_close(out, torch.stack([plain(prompts[2])[-1], plain(prompts[1])[-1]]), rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------- an architecture whose differences lie at the ends of the stack and in the rotation
+
+
+def interleaved_rotation(x, positions, inv_freq, factor):
+    """Channels 2j and 2j + 1 of x [T, heads, d] turn by angle position * inv_freq[j]; cosine and sine times ``factor``."""
+    ang = torch.outer(positions.float(), inv_freq)
+    c, s = ang.cos()[:, None, :] * factor, ang.sin()[:, None, :] * factor
+    a, b = x.float()[..., 0::2], x.float()[..., 1::2]
+    out = torch.empty(x.shape, dtype=torch.float32)
+    out[..., 0::2] = a * c - b * s
+    out[..., 1::2] = b * c + a * s
+    return out.to(x.dtype)
+
+
+def gain_law(shape, generator):
+    """The initial law of a tensor that says so itself: uniform in [0.5, 1.5]."""
+    return torch.rand(shape, generator=generator, device=generator.device) + 0.5
+
+
+@dataclass(frozen=True)
+class GainBiasFfnSpec:
+    """down(silu(gate x) * up x) * gain + bias: a gain drawn by a law of its own and a bias that starts at zero."""
+
+    kind: ClassVar[str] = "gain_bias_ffn"
+    hidden: int
+    inner: int
+
+
+class GainBiasFfn:
+    graph_safe = True  # the product's kernels, then two in-place operations on the output buffer
+
+    def __init__(self, spec, prefix):
+        from nanospec_amd.config.spec import SwiGLUSpec
+        from nanospec_amd.parts import build
+
+        self.spec, self.prefix = spec, prefix
+        self.inner = build("ffn", SwiGLUSpec(spec.hidden, spec.inner), prefix)
+
+    def wanted(self):
+        return {**self.inner.wanted(), self.prefix + "gain": ((self.spec.hidden,), gain_law), self.prefix + "bias": ((self.spec.hidden,), "zeros")}
+
+    def load(self, get, dtype, device):
+        self.inner.load(get, dtype, device)
+        self.gain = get(self.prefix + "gain").to(device=device, dtype=dtype)
+        self.bias = get(self.prefix + "bias").to(device=device, dtype=dtype)
+
+    def forward(self, ctx, x, out=None):
+        out = self.inner.forward(ctx, x, out=out if out is not None else ctx.arena.take((x.shape[0], self.spec.hidden), x.dtype))
+        return out.mul_(self.gain).add_(self.bias)
+
+
+@dataclass(frozen=True)
+class ToyScaledConfig:
+    """Pre-norm blocks as the framework has them, and around them what the Llama decoder does not do: the embedding enters
+    the stream scaled, the logits leave scaled and soft-capped, the rotation pairs neighbouring channels of a part of the
+    head and scales cosine and sine, the feed-forward ends in a gain and a bias."""
+
+    vocab: int
+    width: int
+    depth: int
+    n_head: int
+    n_kv: int
+    d_head: int
+    d_rot: int
+    d_ff: int
+    eps: float
+    rot_factor: float
+    emb_scale: float
+    out_scale: float
+    out_cap: float
+
+    @classmethod
+    def from_hf(cls, cfg, generation_cfg=None):
+        return cls(**{k: cfg[k] for k in cls.__dataclass_fields__})
+
+    def to_hf(self):
+        return dict(architectures=["ToyScaledLM"], model_type="toy_scaled", **self.__dict__)
+
+    def model_spec(self):
+        import math
+
+        from nanospec_amd.config.spec import AttentionSpec, LayerCall, ModelSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec
+
+        norm = RMSNormSpec(self.width, self.eps)
+        rope = RopeSpec(self.d_rot, 1e4, interleaved=True, cos_sin_factor=self.rot_factor)
+        attn = AttentionSpec(self.width, self.n_head, self.n_kv, self.d_head, rope, 1 / math.sqrt(self.d_head))
+        layers = tuple(PreNormBlockSpec(f"blocks.{i}.", norm, attn, norm, GainBiasFfnSpec(self.width, self.d_ff), mixer_norm_name="n1", mixer_prefix="attn.",
+                                        ffn_norm_name="n2", ffn_prefix="ffn.") for i in range(self.depth))
+        return ModelSpec(self.vocab, self.width, "emb", layers, tuple(LayerCall(i) for i in range(self.depth)), norm, "n_out", "head", False,
+                         embed_scale=self.emb_scale, logit_scale=self.out_scale, logit_softcap=self.out_cap)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_an_architecture_with_other_ends_and_another_rotation(tmp_path, dtype):
+    """Registered from this file, nothing in the package changed: interleaved rotation of half a head with a factor on cosine
+    and sine, an embedding scale, a logit scale and soft cap, a part whose tensors name their own initial laws.  The
+    framework writes its folder, finds it by config.json, generates, and replays whole, in portions and token by token
+    (in bfloat16 through the kernels that fuse the rotation into the q/k/v product, and through captured steps)."""
+    from nanospec_amd import SamplingParams, generate, load_model
+    from nanospec_amd.config import register_architecture
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.parts import register
+    from nanospec_amd.weights import write_model_folder
+
+    register("ffn", "gain_bias_ffn", GainBiasFfn)
+    register_architecture("ToyScaledLM", lambda cfg, gen=None: (lambda c: (c, c.model_spec()))(ToyScaledConfig.from_hf(cfg, gen)),
+                          model_type="toy_scaled")
+    c = ToyScaledConfig(vocab=211, width=1024, depth=2, n_head=4, n_kv=2, d_head=32, d_rot=16, d_ff=192, eps=1e-5, rot_factor=0.8,
+                        emb_scale=7.5, out_scale=0.6, out_cap=3.0)
+    folder = write_model_folder(tmp_path / "toy", c, seed=21, dtype=dtype)
+    w = pl.read_safetensors(folder / "model.safetensors")
+    for i in range(c.depth):
+        gain, bias = w[f"blocks.{i}.ffn.gain"].float(), w[f"blocks.{i}.ffn.bias"].float()
+        assert torch.count_nonzero(bias) == 0 and 0.5 <= gain.min() < gain.max() <= 1.5 and gain.std() > 0.2
+        w[f"blocks.{i}.ffn.bias"] = (torch.randn(c.width, generator=torch.Generator().manual_seed(i)) * 0.05).to(dtype)  # a bias that shows
+    from safetensors.torch import save_file
+
+    save_file({k: v.contiguous() for k, v in w.items()}, str(folder / "model.safetensors"))
+    inv = pl.inverse_frequencies(c.d_rot, 1e4, None)
+
+    def plain(tokens):
+        t = len(tokens)
+        pos = torch.arange(t)
+        x = (w["emb"][torch.tensor(tokens)].float() * c.emb_scale).to(dtype)
+        turn = lambda y: torch.cat([interleaved_rotation(y[..., : c.d_rot], pos, inv, c.rot_factor), y[..., c.d_rot :]], -1)
+        for i in range(c.depth):
+            p = f"blocks.{i}."
+            h = pl.rms_norm(x, w[p + "n1"], c.eps)
+            q = turn(pl.linear(h, w[p + "attn.q_proj.weight"]).view(t, c.n_head, c.d_head))
+            k = turn(pl.linear(h, w[p + "attn.k_proj.weight"]).view(t, c.n_kv, c.d_head))
+            v = pl.linear(h, w[p + "attn.v_proj.weight"]).view(t, c.n_kv, c.d_head)
+            x = pl.residual_add(x, pl.linear(pl.causal_attention(q, k, v).reshape(t, -1), w[p + "attn.o_proj.weight"]))
+            h = pl.rms_norm(x, w[p + "n2"], c.eps)
+            f = pl.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+            f = (f * w[p + "ffn.gain"]) + w[p + "ffn.bias"]  # two roundings in the stream's precision, as the part does it
+            x = pl.residual_add(x, f)
+        z = pl.rms_norm(x, w["n_out"], c.eps).float() @ w["head"].float().T * c.out_scale
+        return c.out_cap * torch.tanh(z / c.out_cap)
+
+    def close(ours, ref, what):
+        if dtype == torch.float32:
+            err = ((ours - ref).abs().amax(-1) / ref.abs().amax(-1)).max()
+            assert err < 1e-4, (what, float(err))
+        else:
+            assert ulps_of_row_max(ours, ref).max() <= 8, what
+
+    g = torch.Generator().manual_seed(4)
+    toks = torch.randint(0, c.vocab, (90,), generator=g).tolist()
+    ref = plain(toks)
+    assert ref.abs().max() < c.out_cap and ref.abs().max() > 0.5 * c.out_cap * 0.2  # the cap bounds the logits and is not idle
+    model = load_model(folder, dtype=dtype)
+    rep = Replayer(model, 256, page_size=8)
+    out = rep.step([{"id": "whole", "tokens": toks, "want": list(range(90))}], ["whole"])
+    close(out, ref, "whole")
+    at = 0
+    for n in (40, 20, 2, 9) + (1,) * 19:  # 17 to 128 rows, up to 16 rows, single tokens (captured steps)
+        out = rep.step([{"id": "cut", "tokens": toks[at : at + n], "want": list(range(n))}], [])
+        close(out, ref[at : at + n], f"tokens {at}:{at + n}")
+        at += n
+    assert at == 90 and rep.runner.last_used_graph
+    if dtype == torch.float32:
+        seq = list(toks[:12])
+        for _ in range(5):
+            seq.append(int(plain(seq)[-1].argmax()))
+        assert generate(str(folder), [toks[:12]], SamplingParams(max_tokens=5), dtype="float32", block_size=8) == [seq[12:]]

@@ -92,6 +92,17 @@ def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, link_
     if churned:
         churn(rep.manager)
         rep.scattered = 0
+    holders: dict = {}  # (group, page) -> the requests that have held it
+    real_reserve = rep.manager.reserve
+
+    def reserve(req_id, n):
+        real_reserve(req_id, n)
+        for g, table in enumerate(rep.manager.get(req_id).tables):
+            for page in table:
+                if page is not None and page >= 0:
+                    holders.setdefault((g, page), set()).add(req_id)
+
+    rep.manager.reserve = reserve
     for step, w in zip(steps, where):
         out = rep.step(step["entries"], step["end"])
         if rep.runner.last_used_graph and any(len(e["tokens"]) > 1 for e in step["entries"]):
@@ -109,6 +120,7 @@ def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, link_
     rep.manager.check()
     live = [r for r in rep.manager.live if r != "__pad__"]
     assert not live
+    rep.regranted = sum(1 for who in holders.values() if len(who) > 1)  # pages that two requests held in turn
     return rep
 
 
@@ -134,7 +146,9 @@ def test_schedules_match_plain(tiny_folders, name, dtype, schedule):
         # request held before) between two portions of a request that sits that step out
         steps, where, peak = traces.mixed(seqs, seed=int(schedule[5:] or 5))
         max_tokens = peak  # so few pages that finished requests' pages are handed out again
-    replay(model, steps, where, ref, dtype, max_tokens, page)
+    rep = replay(model, steps, where, ref, dtype, max_tokens, page)
+    if schedule.startswith("mixed"):
+        assert rep.regranted > 0, "no page was handed to a second request: the trace does not test the reuse of pages"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -232,6 +246,10 @@ def test_captured_steps_are_dropped_and_captured_again(tiny_folders, monkeypatch
     assert len(set(shapes)) > 3 and len(shapes) > len(set(shapes)), "shapes were meant to be dropped and captured again"
     widths = [w for _, w in captures]
     assert max(widths) >= 4 * min(widths) and min(widths) < 16, "block tables were meant to start narrow and grow"
+    # the captured steps share their intermediates' memory: all of them together hold less than twice what the largest needs
+    arenas = {id(g.arena): g.arena for g in rep.runner._graphs.values()}
+    assert len(arenas) < len(rep.runner._graphs)
+    assert rep.runner.graph_arena_bytes < 2 * max(a.capacity for a in arenas.values()) + 1
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
@@ -478,6 +496,19 @@ def test_real_shape_slice_matches_plain(llama_1b_slice, dtype, request):
         assert seen == {"unadded": 0, "linked": 0}
 
 
+def plain_logits_at(folder, dtype, toks, places) -> dict:
+    """The plain implementation's logits of one sequence at a few places (the head is applied there only)."""
+    cfg, w = pl.read_config(folder), pl.read_weights(folder, dtype)
+    w = {k: (v if v.dim() == 1 else v.float()) for k, v in w.items()}  # the stored values, converted once
+    x = w["model.embed_tokens.weight"][torch.tensor(toks)].to(dtype)
+    cos, sin = pl.rotation_tables(torch.arange(len(toks)), pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"]))
+    for i in range(cfg["layers"]):
+        x = pl.decoder_layer(x, w, f"model.layers.{i}.", cfg, cos, sin)
+    head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
+    ref = pl.rms_norm(x[places], w["model.norm.weight"], cfg["eps"]).float() @ head.T
+    return {p: ref[i] for i, p in enumerate(places)}
+
+
 @pytest.mark.parametrize("slice_k", [8192, 2048])
 def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch, slice_k):
     """A model that keeps the re-laid matrices only.  A prompt portion of 1,100 tokens, launched kernel by kernel: every
@@ -493,16 +524,9 @@ def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch, slice_k):
     monkeypatch.setattr(linear, "PLAIN_SLICE_K", slice_k)
 
     folder, dtype = llama_1b_slice, torch.bfloat16
-    cfg, w = pl.read_config(folder), pl.read_weights(folder, dtype)
-    w = {k: (v if v.dim() == 1 else v.float()) for k, v in w.items()}  # the stored values, converted once
     toks = random_tokens(2010, 128256, 5)
     places = [0, 1, 511, 767, 1099, 1100, 1500, 1899, 1900, 1999, 2000, 2003, 2009]
-    x = w["model.embed_tokens.weight"][torch.tensor(toks)].to(dtype)
-    cos, sin = pl.rotation_tables(torch.arange(len(toks)), pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"]))
-    for i in range(cfg["layers"]):
-        x = pl.decoder_layer(x, w, f"model.layers.{i}.", cfg, cos, sin)
-    ref = pl.rms_norm(x[places], w["model.norm.weight"], cfg["eps"]).float() @ w["lm_head.weight"].T
-    at = {p: ref[i] for i, p in enumerate(places)}
+    at = plain_logits_at(folder, dtype, toks, places)
     model = load_model(folder, dtype=dtype, layouts="tiled")
     calls = {"untile": 0, "rows": 0}
     real_untile, real_rows = ops.untile, ops.linear_rows
@@ -530,6 +554,56 @@ def test_many_rows_with_one_weight_layout(llama_1b_slice, monkeypatch, slice_k):
     for p in range(2000, 2010):
         step(p, p + 1)
     rep.manager.check()
+
+
+def test_long_inner_sizes_never_reach_the_library_in_one_piece(llama_1b_slice, monkeypatch):
+    """Both layouts kept, and the longest inner size that the library takes in one piece set below the down-projection's
+    (8,192 here).  A portion of 1,100 tokens launched kernel by kernel: the down-projection goes to the library in slices
+    summed in 32-bit; the last layer's, which does not end in the stream, through the many-row kernel.  A captured step of
+    800 tokens: the many-row kernel both times.  Every other product stays with the library, and none of the library's
+    products runs over more than the bound."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.kernels import ops
+    from nanospec_amd.loader import load_model
+    from nanospec_amd.parts import linear
+
+    monkeypatch.setattr(linear, "LIBRARY_MAX_K", 4096)
+    monkeypatch.setattr(linear, "PLAIN_SLICE_K", 4096)
+    folder, dtype = llama_1b_slice, torch.bfloat16
+    toks = random_tokens(2010, 128256, 6)
+    places = [0, 700, 1099, 1100, 1899, 1900, 2000, 2009]
+    at = plain_logits_at(folder, dtype, toks, places)
+    model = load_model(folder, dtype=dtype, layouts="both")
+    seen = {"library": [], "rows": []}
+    real_lib, real_rows = linear.library_product, ops.linear_rows
+    monkeypatch.setattr(linear, "library_product", lambda x, w_t, **k: (seen["library"].append((x.shape[1], k.get("into") is not None and k["into"].dtype == torch.float32)), real_lib(x, w_t, **k))[1])
+    monkeypatch.setattr(ops, "linear_rows", lambda x, w, **k: (seen["rows"].append(w.k), real_rows(x, w, **k))[1])
+    rep = Replayer(model, 2048, page_size=16)
+
+    def step(s, e):
+        wants = [p - s for p in places if s <= p < e]
+        out = rep.step([{"id": "a", "tokens": toks[s:e], "want": wants}], [])
+        if wants:
+            check(out, torch.stack([at[s + i] for i in wants]), dtype, f"tokens {s}:{e}")
+
+    step(0, 1100)
+    assert not rep.runner.last_used_graph
+    # q/k/v, o and gate/up of both layers in one piece; the first layer's down-projection in two slices into a 32-bit sum
+    assert sorted(seen["library"]) == [(2048, False)] * 6 + [(4096, True)] * 2, seen
+    assert seen["rows"] == [8192], seen
+    seen["library"].clear(), seen["rows"].clear()
+    step(1100, 1900)
+    assert rep.runner.last_used_graph
+    # (the step ran twice: once before its capture and once while captured)
+    assert sorted(seen["library"]) == [(2048, False)] * 12 and seen["rows"] == [8192] * 4, seen
+    step(1900, 2000)
+    for p in range(2000, 2010):
+        step(p, p + 1)
+    assert max(k for k, _ in seen["library"]) <= 4096
+    rep.manager.check()
+    with pytest.raises(ops.KernelRefused):
+        x = torch.zeros((256, 8192), dtype=dtype, device="cuda")
+        real_lib(x, torch.zeros((8192, 64), dtype=dtype, device="cuda"))
 
 
 @pytest.fixture(scope="module")

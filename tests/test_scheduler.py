@@ -150,8 +150,8 @@ def test_a_prompt_advances_although_the_decoding_requests_fill_the_budget():
 
 def test_decoding_rows_count_as_the_engine_pads_them():
     """The engine rounds the rows of decoding requests up to a captured step's size and says so through ``decode_rows_cost``:
-    the budget is then charged for the padded rows, so a step with its padding stays within it, and when not all decoding
-    requests fit it takes as many as fit with their padding."""
+    the budget is charged for the padded rows where they fit it, so that such a step stays within it with its padding, and for
+    the rows as they are where they do not."""
     buckets = (1, 2, 4, 8)
     cost = lambda n: next((b for b in buckets if b >= n), n) if n else 0
     s = Scheduler(manager(256, 4), max_admit=16, max_step_tokens=32)
@@ -162,19 +162,26 @@ def test_decoding_rows_count_as_the_engine_pads_them():
     s.add(req(5, 100, max_tokens=2))
     work = run_step(s)
     assert ids(work) == [(i, 1) for i in range(5)] + [(5, 24)]  # five rows are padded to eight: 24 of 32 are left
-    # a budget of six: five rows would be padded to eight, so four go (padded to four) and the prompt has the rest
+    # a budget of six: five rows padded to eight do not fit, so they are charged as the five they are (nobody who fits is
+    # left out because of padding) and the prompt has the one token that is left
     s = Scheduler(manager(256, 4), max_admit=16, max_step_tokens=6)
     s.decode_rows_cost = cost
     for i in range(5):
         s.add(req(i, 1, max_tokens=40))
-    run_step(s), run_step(s)  # prompts of one token: two steps under this budget
+    run_step(s)
     s.add(req(5, 100, max_tokens=2))
     for _ in range(6):
-        work = run_step(s)
-        n_dec = sum(1 for w in work if w.req.id != 5)
-        assert cost(n_dec) + sum(w.n for w in work if w.req.id == 5) <= 6
-        assert any(w.req.id == 5 for w in work)
-    assert max(len(r.out_tokens) for r in s.running if r.id != 5) - min(len(r.out_tokens) for r in s.running if r.id != 5) <= 1
+        assert ids(run_step(s)) == [(i, 1) for i in range(5)] + [(5, 1)]
+    # a budget that is no multiple of the padding: 20 decoding requests under 24 all advance (32 padded rows do not fit),
+    # where a budget of 40 charges the 32 and leaves a prompt 8
+    for budget, portion in ((24, 4), (40, 8)):
+        s = Scheduler(manager(1024, 4, slots=32), max_admit=32, max_step_tokens=budget)
+        s.decode_rows_cost = lambda n: next((b for b in (1, 2, 4, 8, 16, 32) if b >= n), n) if n else 0
+        for i in range(20):
+            s.add(req(i, 1, max_tokens=40))
+        run_step(s)
+        s.add(req(20, 100, max_tokens=2))
+        assert ids(run_step(s)) == [(i, 1) for i in range(20)] + [(20, portion)]
 
 
 def test_preemption_when_pages_run_out():
