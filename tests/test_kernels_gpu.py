@@ -779,3 +779,59 @@ def test_sample_top_k_top_p(vocab, spread):
                 cdf = torch.cumsum(torch.exp(ref_lp.double()), 0)
                 assert abs(float(cdf[got]) - float(cdf[ref])) < 2e-3, (r, uu, got, ref)
                 assert abs(float(slp[r]) - float(ref_lp[ref])) < 1e-2
+
+
+# ------------------------------------------------------------------------------------------------ the largest sizes
+
+
+def _big(n, k, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    return (torch.randn(n, k, dtype=torch.float32, device=DEV, generator=g) * 0.05).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("n,k", [(8192, 28672), (28672, 8192)])
+def test_products_at_the_largest_feed_forward_sizes(n, k):
+    """The hand-written products at an inner size and at an output width of 28,672 (the Llama-3.1-70B feed-forward): the
+    streaming kernel at 1, 8 and 16 rows, the 17-to-128-row kernel at 64 and 128 rows with K in its planned ranges, the
+    many-row kernel at 300 rows, the gated forms, and the product that ends in the residual stream and feeds the next
+    norm; each against the 32-bit product of the same bfloat16 values."""
+    ops = _ops()
+    w, w2 = _big(n, k, 1), _big(n, k, 2)
+    wt, wt2 = ops.TiledWeight(w), ops.TiledWeight(w2)
+    wf, w2f = w.cpu().float(), w2.cpu().float()
+    x_all = (torch.randn(300, k, dtype=torch.float32, device=DEV, generator=torch.Generator(device=DEV).manual_seed(3))).to(torch.bfloat16)
+    ref_all = x_all.cpu().float() @ wf.T
+    for m in (1, 8, 16):
+        x, ref = x_all[:m], ref_all[:m]
+        assert ulps_of_row_max(ops.linear_tiled(x, wt).cpu(), ref).max() <= 1.0, m
+        u = x.cpu().float() @ w2f.T
+        assert ulps_of_row_max(ops.linear_tiled(x, wt, w2=wt2).cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0, m
+    for m in (64, 128):
+        x, ref = x_all[:m], ref_all[:m]
+        ksplit, nt = ops.wide_plan(n, k, m)
+        out = ops.linear_wide(x, wt, ksplit=ksplit, nt=nt)
+        assert ulps_of_row_max(out.cpu(), ref).max() <= 1.0, (m, ksplit, nt)
+        part = ops.linear_wide(x, wt, ksplit=max(2, ksplit), nt=1, defer=True)
+        assert ulps_of_row_max(ops.reduce_partial(part).cpu(), ref).max() <= 1.0, m
+    u = x_all[:64].cpu().float() @ w2f.T
+    act = ops.linear_wide(x_all[:64], wt, w2=wt2, ksplit=1, nt=1)
+    assert ulps_of_row_max(act.cpu(), ref_all[:64] * torch.sigmoid(ref_all[:64]) * u).max() <= 1.0
+    assert ulps_of_row_max(ops.linear_rows(x_all, wt).cpu(), ref_all).max() <= 1.0
+    u = x_all.cpu().float() @ w2f.T
+    assert ulps_of_row_max(ops.linear_rows(x_all, wt, w2=wt2, ksplit=1, nt=2).cpu(), ref_all * torch.sigmoid(ref_all) * u).max() <= 1.0
+    # resid += x W^T with the next norm's inputs as by-products, 8 rows
+    m = 8
+    resid = (torch.randn(m, n, device=DEV) * 2).to(torch.bfloat16)
+    w_next = (1 + 0.1 * torch.randn(n, device=DEV)).to(torch.bfloat16)
+    before = resid.clone()
+    pre = ops.linear_resid_norm(x_all[:m], wt, resid, w_next, 1e-5)
+    want = (before.cpu().float() + ref_all[:m].to(torch.bfloat16).float()).to(torch.bfloat16)
+    assert ulps_of_row_max(resid.cpu(), want.float()).max() <= 1.0
+    torch.testing.assert_close(pre.ssq.sum(-1).cpu(), (resid.cpu().float() ** 2).sum(-1), rtol=1e-4, atol=0)
+    assert torch.equal(pre.x.cpu(), (resid.cpu().float() * w_next.cpu().float()).to(torch.bfloat16))
+    # a matrix copied back into plain rows, whole and in slices of its inner size
+    plain = torch.empty_like(w)
+    assert torch.equal(ops.untile(wt, plain), w)
+    piece = torch.empty((n, 7168 if k > 8192 else 2048), dtype=torch.bfloat16, device=DEV)
+    width = piece.shape[1]
+    assert torch.equal(ops.untile(wt, piece, width, 2 * width), w[:, width : 2 * width])

@@ -747,3 +747,214 @@ def test_benchmark_shape_slice_matches_plain(llama_8b_slice, dtype):
     step([(r, 1, [0]) for r in first8[1:] + rest] + [("r64", 40, [0, 39])])
     assert all(at[r] == lengths[r] for r in lengths if r != "r0") and at["r0"] == 304
     rep.manager.check()
+
+
+class PlainRows:
+    """The plain implementation's logits at chosen (request, position) places of many sequences: every sequence runs
+    whole through the plain layers once (matrices held as 32-bit tensors of the stored values, converted once), the last
+    norm and the head only at the places asked for."""
+
+    _stored: dict = {}  # folder -> its tensors in 32-bit (the stored values; shared by the runs in both precisions)
+
+    def __init__(self, folder, dtype, seqs: dict) -> None:
+        self.cfg = cfg = pl.read_config(folder)
+        if str(folder) not in self._stored:
+            self._stored.clear()  # one model's worth of memory at a time
+            self._stored[str(folder)] = pl.read_weights(folder, torch.float32)
+        # vectors (norm weights) in the run's precision, which decides how the norm rounds
+        self.w = w = {k: (v.to(dtype) if v.dim() == 1 else v) for k, v in self._stored[str(folder)].items()}
+        inv = pl.inverse_frequencies(cfg["head_dim"], cfg["theta"], cfg["scaling"])
+        self.hidden = {}
+        for r, toks in seqs.items():
+            x = w["model.embed_tokens.weight"][torch.tensor(toks)].to(dtype)
+            cos, sin = pl.rotation_tables(torch.arange(len(toks)), inv)
+            for i in range(cfg["layers"]):
+                x = pl.decoder_layer(x, w, f"model.layers.{i}.", cfg, cos, sin)
+            self.hidden[r] = x
+
+    def __call__(self, places) -> torch.Tensor:
+        x = torch.stack([self.hidden[r][p] for r, p in places])
+        return pl.rms_norm(x, self.w["model.norm.weight"], self.cfg["eps"]).float() @ self.w["lm_head.weight"].float().T
+
+
+class Stepper:
+    """Feeds sequences through a Replayer in the steps a test names and compares the wanted logits with ``PlainRows``."""
+
+    def __init__(self, rep, seqs, plain, dtype) -> None:
+        self.rep, self.seqs, self.plain, self.dtype = rep, seqs, plain, dtype
+        self.at = {r: 0 for r in seqs}
+
+    def __call__(self, parts, end=(), graph=None):
+        """parts: (request, tokens it brings, places among them whose logits are compared); ``graph``: the (rows, tokens)
+        of the captured step that must have run, or False for a step launched kernel by kernel."""
+        entries, places = [], []
+        for r, n, wants in parts:
+            entries.append({"id": r, "tokens": self.seqs[r][self.at[r] : self.at[r] + n], "want": list(wants)})
+            places += [(r, self.at[r] + i) for i in wants]
+            self.at[r] += n
+        out = self.rep.step(entries, list(end))
+        if graph is False:
+            assert not self.rep.runner.last_used_graph
+        elif graph is not None:
+            assert self.rep.runner.last_used_graph and graph in self.rep.runner._graphs, (graph, list(self.rep.runner._graphs))
+        if places:
+            check(out, self.plain(places), self.dtype, str([(r, n) for r, n, _ in parts][:4]))
+        else:
+            assert out is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_benchmark_shape_steps_of_many_rows_match_plain(llama_8b_slice, dtype):
+    """Steps of more than 128 rows at the benchmark's layer sizes, where other code runs than below (the library's
+    products, sums into the stream by the library, norms of their own), against the plain implementation: decoding with
+    200 live requests (the captured step of 208 rows) and a captured step of 32 decode rows beside a prompt portion of
+    480 tokens, replayed with new tokens."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.loader import load_model
+
+    folder = llama_8b_slice
+    vocab = pl.read_config(folder)["vocab"]
+    lengths = {**{f"d{i}": 3 + i % 6 + 4 for i in range(200)}, "p": 2 * 480 + 3}
+    seqs = {r: random_tokens(n, vocab, 8100 + i) for i, (r, n) in enumerate(lengths.items())}
+    plain = PlainRows(folder, dtype, seqs)
+    model = load_model(folder, dtype=dtype)
+    rep = Replayer(model, 201 * 64 + 1024, page_size=16, max_live=201)
+    step = Stepper(rep, seqs, plain, dtype)
+    rows = [f"d{i}" for i in range(200)]
+    for at in range(0, 200, 50):  # the prompts, fifty requests a step
+        step([(r, lengths[r] - 4, [lengths[r] - 5] if r in ("d0", "d57", "d199") else []) for r in rows[at : at + 50]])
+    every = [0] if dtype == torch.bfloat16 else []
+    shown = {"d0", "d1", "d57", "d128", "d129", "d199"}  # (the 32-bit head over 200 rows takes its time: a few rows there)
+    for _ in range(2):
+        step([(r, 1, [0] if (every or r in shown) else []) for r in rows], graph=(208, 0))
+    # 32 decode rows beside 480 prompt tokens: 512 rows in one captured step, twice
+    for k in range(2):
+        step([(r, 1, [0]) for r in rows[:32]] + [("p", 480, [0, 479])], graph=(32, 480), end=rows if k else ())
+    step([("p", 3, [0, 1, 2])], end=["p"])
+    rep.manager.check()
+
+
+# ------------------------------------------------------------------------------------------------ the target model, whole
+
+
+@pytest.fixture(scope="module")
+def llama_1b_full(tmp_path_factory):
+    """The Llama-3.2-1B shape at its full depth: 16 layers of width 2048, 32 heads over 8 key/value heads of 64,
+    feed-forward 8192, vocabulary 128256, the head tied to the embedding, llama3 scaling with factor 32; random weights."""
+    from nanospec_amd.config import LlamaConfig
+    from nanospec_amd.weights import write_model_folder
+
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8, head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0,
+               max_position_embeddings=131072, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    return write_model_folder(tmp_path_factory.mktemp("llama1b_full") / "m", LlamaConfig.from_hf(cfg), seed=16, dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_llama_1b_at_full_depth_matches_plain(llama_1b_full, dtype):
+    """reference tests/test_correctness.py:68-80, at the depth of the model itself: sixteen layers of rounding on top of
+    each other, the tied head of 128,256 rows after them.  One request whole; one with its last 32 tokens decoded one by
+    one (captured steps); a third joins as a portion beside a decoded token, goes on with two tokens beside the next, and
+    decodes beside it."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.loader import load_model
+
+    folder = llama_1b_full
+    seqs = {"a": random_tokens(100, 128256, 41), "b": random_tokens(100, 128256, 42), "c": random_tokens(45, 128256, 43)}
+    plain = PlainRows(folder, dtype, seqs)
+    model = load_model(folder, dtype=dtype)
+    assert len(model.layers) == 16 and model.spec.tie_head
+    rep = Replayer(model, 4 * 128, page_size=16)
+    step = Stepper(rep, seqs, plain, dtype)
+    step([("a", 100, [0, 1, 31, 63, 64, 98, 99])], end=["a"], graph=False)
+    step([("b", 68, [0, 67])])
+    for p in range(68, 100):
+        if p == 80:
+            step([("b", 1, [0]), ("c", 37, [0, 36])])
+        elif p == 81:
+            step([("b", 1, [0]), ("c", 2, [0, 1])])
+        elif p < 88:
+            step([("b", 1, [0])] + ([("c", 1, [0])] if p > 81 else []))
+        else:
+            step([("b", 1, [0])], graph=(1, 0), end=["b"] if p == 99 else [])
+    assert step.at == {"a": 100, "b": 100, "c": 45}
+    rep.runner.release("c")
+    rep.manager.check()
+
+
+# ------------------------------------------------------------------------------------------------ the largest layer sizes
+
+
+@pytest.fixture(scope="module")
+def llama_70b_layer(tmp_path_factory):
+    """Two layers of the Llama-3.1-70B shape (width 8192, 64 heads over 8 key/value heads of 128, feed-forward 28672,
+    llama3 scaling with factor 8) with a vocabulary of 512, so that the plain implementation's head costs nothing.  (Two,
+    because a layer's last product is handed to the next layer's norm in other forms than to the norm before the head.)"""
+    from nanospec_amd.config import LlamaConfig
+    from nanospec_amd.weights import write_model_folder
+
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=512, hidden_size=8192, intermediate_size=28672,
+               num_hidden_layers=2, num_attention_heads=64, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-5, rope_theta=500000.0,
+               max_position_embeddings=131072, tie_word_embeddings=False,
+               rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    return write_model_folder(tmp_path_factory.mktemp("llama70b") / "m", LlamaConfig.from_hf(cfg), seed=70, dtype=torch.bfloat16)
+
+
+_PLAIN_70B = {}
+
+
+@pytest.mark.parametrize("layouts", ["tiled", "both"])
+def test_the_largest_layer_sizes_match_plain(llama_70b_layer, layouts, monkeypatch):
+    """reference tests/test_backends.py:25-71 runs its kernels at the real head shape; here a whole layer at the largest
+    shape the benchmark names, with only the re-laid matrices kept and with both layouts: a step of 1,100 tokens launched
+    kernel by kernel (the library over plain copies or plain rows; the down-projection's inner size of 28,672 in four
+    slices summed in 32-bit), a captured step of 800 tokens (the many-row kernel for what the library is kept from),
+    decoding with 8 and with 64 live requests, and 63 decode rows beside a new prompt."""
+    from nanospec_amd.engine.replay import Replayer
+    from nanospec_amd.kernels import ops
+    from nanospec_amd.loader import load_model
+    from nanospec_amd.parts import linear
+
+    folder, dtype = llama_70b_layer, torch.bfloat16
+    lengths = {"p": 1903, **{f"r{i}": 4 + i % 7 + 5 for i in range(64)}, "q": 40}
+    seqs = {r: random_tokens(n, 512, 7700 + i) for i, (r, n) in enumerate(lengths.items())}
+    if "plain" not in _PLAIN_70B:
+        _PLAIN_70B["plain"] = PlainRows(folder, dtype, seqs)
+    plain = _PLAIN_70B["plain"]
+    model = load_model(folder, dtype=dtype, layouts=layouts)
+    seen = {"library": [], "rows": 0, "untile": 0}
+    real_lib, real_rows, real_untile = linear.library_product, ops.linear_rows, ops.untile
+    monkeypatch.setattr(linear, "library_product", lambda x, w_t, **k: (seen["library"].append(x.shape[1]), real_lib(x, w_t, **k))[1])
+    monkeypatch.setattr(ops, "linear_rows", lambda *a, **k: (seen.__setitem__("rows", seen["rows"] + 1), real_rows(*a, **k))[1])
+    monkeypatch.setattr(ops, "untile", lambda *a, **k: (seen.__setitem__("untile", seen["untile"] + 1), real_untile(*a, **k))[1])
+    rep = Replayer(model, 2048 + 66 * 64, page_size=16, max_live=66)
+    step = Stepper(rep, seqs, plain, dtype)
+    step([("p", 1100, [0, 1, 640, 1099])], graph=False)
+    # q/k/v, o, gate/up of both layers in one piece each and the first layer's down-projection in four slices of 7,168,
+    # whichever layouts are kept; the last layer's, which does not end in the stream, through the many-row kernel
+    assert sorted(seen["library"]) == [7168] * 4 + [8192] * 6, seen
+    assert seen["rows"] == 1 and seen["untile"] == (12 if layouts == "tiled" else 0), seen
+    seen["library"].clear()
+    seen["rows"] = 0
+    step([("p", 800, [0, 799])], graph=(0, 832))
+    # (the step ran twice, before and during its capture) the down-projection through the many-row kernel; with only the
+    # re-laid matrices every product, with both layouts the other three through the library
+    if layouts == "tiled":
+        assert seen["library"] == [] and seen["rows"] == 2 * 2 * 4, seen
+    else:
+        assert sorted(seen["library"]) == [8192] * 12 and seen["rows"] == 2 * 2, seen
+    step([("p", 3, [0, 1, 2])], end=["p"])
+    first8 = [f"r{i}" for i in range(8)]
+    step([(r, lengths[r] - 5, [lengths[r] - 6]) for r in first8])
+    for _ in range(2):
+        step([(r, 1, [0]) for r in first8], graph=(8, 0))
+    rest = [f"r{i}" for i in range(8, 64)]
+    step([(r, lengths[r] - 3, [lengths[r] - 4]) for r in rest])
+    for _ in range(2):
+        step([(r, 1, [0]) for r in first8 + rest], graph=(64, 0))
+    step([(r, 1, [0]) for r in first8[1:] + rest] + [("q", 40, [0, 39])])
+    assert max(seen["library"], default=0) <= linear.LIBRARY_MAX_K
+    rep.manager.check()
