@@ -23,6 +23,7 @@
 // With splits > 1 the keys of a tile are cut into `splits` contiguous ranges of whole 32-key blocks;
 // each range writes its un-normalised output, maximum and sum, and a second small kernel joins them.
 #include "common.h"
+#include <type_traits>
 
 #if !defined(NS_HEAD_DIM) || !defined(NS_PAGE_SIZE)
 #error "compile with -DNS_HEAD_DIM=<multiple of 16> -DNS_PAGE_SIZE=<power of two from 4>"
@@ -55,6 +56,8 @@ struct AttnParams {
   const int* tiles;   // [n_tiles][TILE_INTS]
   const int* block_table;
   int q_stride, table_stride, n_tiles, heads, kv_heads, hp, splits, window;
+  int near;          // every byte of the key pool and of the value pool lies within 4 GiB of its start, a page's id and a
+                     // page's bytes are below 2^24: byte offsets are then 32-bit and one 24-bit multiply-add each
   float scale_log2;  // softmax scale * log2(e)
 };
 
@@ -464,6 +467,16 @@ __device__ __forceinline__ float max_over_lane_rows(float x) {
   return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
 }
 
+// In a stretch of straight code: N times one matrix instruction and then V vector instructions, in that order of issue.
+#ifndef NS_VALU_PER_MFMA
+#define NS_VALU_PER_MFMA 5
+#endif
+#define NS_STAGE(N, V)                                        \
+  _Pragma("unroll") for (int sg_ = 0; sg_ < (N); ++sg_) {     \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+    __builtin_amdgcn_sched_group_barrier(0x002, (V), 0);      \
+  }
+
 constexpr bool SHARED_OK = WIDE && PS >= 8 && HD <= 128;  // larger heads do not fit two waves' registers per SIMD
 constexpr int KROW = HD + 16;               // elements of a key's row in LDS
 constexpr int VROW = 32 + 16;               // elements of a channel's row in LDS
@@ -555,6 +568,8 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       for (int dt = 0; dt < DT; ++dt) o[u][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
+    const bf16_t one = (bf16_t)1.0f;
+    const bf16x8 ones = {one, one, one, one, one, one, one, one};
     // This thread's pieces of a block: piece r of the keys is 8 channels of one key, piece r of the values 8 keys of
     // one channel.
     int k_key[PER_THREAD], k_off[PER_THREAD], k_lds[PER_THREAD];
@@ -635,7 +650,10 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
     // One block of 32 keys for this wave's two 16-token columns.  The order of the source is the order of issue: the
     // matrix instructions of one column run while the vector unit does the soft-max arithmetic of the other
     // (scores u0, scores u1 | soft-max u0 under them, sums u0 | soft-max u1 under them, sums u1).
-    auto block = [&](int buf, int kb) {
+    auto block = [&](int buf, int kb, auto full_tag) {
+      // full_tag: every key of the block is seen by every token of the tile (known when the loop was entered), so the
+      // code of such blocks holds no masks at all; the few blocks at the ends of a tile's keys run the other form
+      constexpr bool FULL = decltype(full_tag)::value;
       const int key_base = kb * 32;
       bf16x8 kf[2][NQ];
 #pragma unroll
@@ -653,43 +671,34 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
           s[u][t] = acc;
         }
       // s[u][t][j] is key key_base + 8 g + 4 t + j of column c
-      const bool full = key_base + 31 <= full_hi && key_base >= full_lo;  // no masks needed (uniform over the workgroup)
       bf16x8 pf[2];
       auto soften = [&](int u) {
         float mx = -INFINITY;
-        if (full) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][t][j]);
-        } else {
+        if (!FULL) {
 #pragma unroll
           for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               const int key = key_base + g * 8 + t * 4 + j;
-              const float v = (key >= lo[u] && key <= pos[u]) ? s[u][t][j] : -INFINITY;
-              s[u][t][j] = v;
-              mx = fmaxf(mx, v);
+              s[u][t][j] = (key >= lo[u] && key <= pos[u]) ? s[u][t][j] : -INFINITY;
             }
         }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][t][j]);
         mx = max_over_lane_rows(mx);
         // m[u] is the running maximum of the raw scores (the scale is positive); p = 2^((s - m) scale log2 e)
         const float m_new = fmaxf(m[u], mx);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float m_safe = (!FULL && m_new == -INFINITY) ? 0.f : m_new;  // (a full block's maximum is a score)
         const bool moved = m_new != m[u];
         const float alpha = fast_exp2((m[u] - m_safe) * a.scale_log2);
         const float shift = -m_safe * a.scale_log2;
         m[u] = m_new;
-        float psum = 0.f;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float p = fast_exp2(fmaf(s[u][t][j], a.scale_log2, shift));
-            psum += p;
-            pf[u][t * 4 + j] = (bf16_t)p;
-          }
+          for (int j = 0; j < 4; ++j) pf[u][t * 4 + j] = (bf16_t)fast_exp2(fmaf(s[u][t][j], a.scale_log2, shift));
         if (__any(moved)) {  // the maximum settles early in long rows; rescaling is skipped from then on
           lsum[u] *= alpha;
 #pragma unroll
@@ -697,14 +706,26 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
 #pragma unroll
             for (int j = 0; j < 4; ++j) o[u][dt][j] *= alpha;
         }
-        lsum[u] += psum;
       };
+#ifdef NS_VONCE
+      bf16x8 vfr[DT];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vfr[dt] = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
+#endif
       auto weigh = [&](int u) {
+        // the block's sum of weights by one more matrix instruction against ones: every row of the result is the sum over
+        // the 32 keys of the weights as the value products see them (rounded to bfloat16), for this lane's column
+        const f32x4 tot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[u], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
+#ifdef NS_VONCE
+          const bf16x8 vf = vfr[dt];
+#else
           const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
+#endif
           o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
         }
+        lsum[u] += tot[0];
       };
       soften(0);
       weigh(0);
@@ -730,20 +751,153 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
     // every barrier; the second may have no block in the last round.
     auto round = [&](bf16x8(&kr_far)[PER_THREAD], bf16x8(&vr_far)[PER_THREAD], int(&kp_far)[PER_THREAD], int(&vp_far)[PER_THREAD],
                      const bf16x8(&kr_next)[PER_THREAD], const bf16x8(&vr_next)[PER_THREAD], int(&kp_next)[PER_THREAD],
-                     int(&vp_next)[PER_THREAD], int it) {
+                     int(&vp_next)[PER_THREAD], int it, auto full_tag) {
       const int kb = kb0 + it;
       const int buf = it & 1;
       if (kb + 2 < kb1) {
         if (kb + 3 < kb1) fetch_pages(kp_next, vp_next, kb + 3);  // the set that block it + 1's loads were issued from
         fetch(kr_far, vr_far, kp_far, vp_far, kb + 2);
       }
-      if (head_ok && kb < kb1) block(buf, kb);
+      if (head_ok && kb < kb1) block(buf, kb, full_tag);
       if (kb + 1 < kb1) put(kr_next, vr_next, buf ^ 1);
       __syncthreads();
     };
-    for (int it = 0; it < steps; it += 2) {
-      round(kst[0], vst[0], kps[0], vps[0], kst[1], vst[1], kps[1], vps[1], it);
-      if (it + 1 < steps) round(kst[1], vst[1], kps[1], vps[1], kst[0], vst[0], kps[0], vps[0], it + 1);
+    // A round of the long middle of a tile's keys, where nothing needs asking: the block is seen wholly by every token, all
+    // four waves have a head, and the blocks whose ids and data are asked for lie inside the tile's keys and are not the
+    // last.  Its matrix instructions and its vector arithmetic are laid side by side, stage by stage, because the matrix
+    // unit runs a wave's instruction while the wave issues vector instructions that do not wait for it:
+    //   1  the next loads are issued               beside  the scores of the first column
+    //   2  the first column's soft-max weights     beside  the scores of the second column
+    //   3  the second column's soft-max weights    beside  the first column's weighted values
+    //   4  the next block goes into LDS            beside  the second column's weighted values
+    // (a column's sums are rescaled between two stages, and only when its maximum moved).
+    auto steady = [&](bf16x8(&kr_far)[PER_THREAD], bf16x8(&vr_far)[PER_THREAD], int(&kp_far)[PER_THREAD], int(&vp_far)[PER_THREAD],
+                      const bf16x8(&kr_next)[PER_THREAD], const bf16x8(&vr_next)[PER_THREAD], int(&kp_next)[PER_THREAD],
+                      int(&vp_next)[PER_THREAD], int it, auto near_tag) {
+      constexpr bool NEAR = decltype(near_tag)::value;
+      const int kb = kb0 + it, buf = it & 1;
+      const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+      // ---- 1
+#pragma unroll
+      for (int r = 0; r < PER_THREAD; ++r) {
+        kp_next[r] = table[(kb + 3) * PPB + k_slot[r]];
+        vp_next[r] = table[(kb + 3) * PPB + v_slot[r]];
+      }
+#pragma unroll
+      for (int r = 0; r < PER_THREAD; ++r) {
+        if (NEAR) {
+          const unsigned page_bytes = (unsigned)kv_page * 2;
+          const unsigned ko = __umul24((unsigned)kp_far[r], page_bytes) + (unsigned)k_const[r] * 2;
+          const unsigned vo = __umul24((unsigned)vp_far[r], page_bytes) + (unsigned)v_const[r] * 2;
+          kr_far[r] = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(a.k_cache) + ko);
+          vr_far[r] = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(a.v_cache) + vo);
+        } else {
+          kr_far[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)kp_far[r] * kv_page + k_const[r]);
+          vr_far[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)vp_far[r] * kv_page + v_const[r]);
+        }
+      }
+      bf16x8 kf[2][NQ];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) kf[t][i] = *reinterpret_cast<const bf16x8*>(&lk[buf][(16 * t + c) * KROW + 32 * i + 8 * g]);
+      f32x4 s[2][2];
+      auto scores = [&](int u) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) s[u][t] = zero4;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) s[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][i], qw[u][i], s[u][t], 0, 0, 0);
+      };
+      bf16x8 pf[2];
+      float alpha[2];
+      auto soften = [&](int u) -> bool {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][t][j]);
+        mx = max_over_lane_rows(mx);
+        const float m_new = fmaxf(m[u], mx);
+        const bool moved = m_new != m[u];
+        alpha[u] = fast_exp2((m[u] - m_new) * a.scale_log2);
+        const float shift = -m_new * a.scale_log2;
+        m[u] = m_new;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) pf[u][t * 4 + j] = (bf16_t)fast_exp2(fmaf(s[u][t][j], a.scale_log2, shift));
+        return __any(moved);
+      };
+      auto rescale = [&](int u) {
+        lsum[u] *= alpha[u];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[u][dt][j] *= alpha[u];
+      };
+      auto weigh = [&](int u) {
+        const f32x4 tot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[u], zero4, 0, 0, 0);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&lv[buf][(16 * dt + c) * VROW + 8 * g]);
+          o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o[u][dt], 0, 0, 0);
+        }
+        lsum[u] += tot[0];
+      };
+      scores(0);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- 2
+      scores(1);
+      const bool moved0 = soften(0);
+      NS_STAGE(8, NS_VALU_PER_MFMA)
+      asm volatile("" : "+v"(pf[0]));  // the weights are formed here, beside the matrix instructions, not where they are used
+      __builtin_amdgcn_sched_barrier(0);
+      if (moved0) rescale(0);
+      // ---- 3
+      weigh(0);
+      const bool moved1 = soften(1);
+      NS_STAGE(9, NS_VALU_PER_MFMA)
+      asm volatile("" : "+v"(pf[1]));
+      __builtin_amdgcn_sched_barrier(0);
+      if (moved1) rescale(1);
+      // ---- 4
+      weigh(1);
+#pragma unroll
+      for (int r = 0; r < PER_THREAD; ++r)
+        if (mine[r]) {
+          *reinterpret_cast<bf16x8*>(&lk[buf ^ 1][k_lds[r]]) = kr_next[r];
+          *reinterpret_cast<bf16x8*>(&lv[buf ^ 1][v_lds[r]]) = vr_next[r];
+        }
+      __syncthreads();
+    };
+
+    // The first blocks of this set's range that every token of the tile sees wholly (an even number of them: rounds go in
+    // pairs, one per register set) run the form without masks.  Both sets pass a barrier in every round, whichever form
+    // a round takes.
+    const int seen_whole = a.window > 0 ? 0 : min(max((full_hi + 1) / 32 - kb0, 0), max(kb1 - kb0, 0)) & ~1;
+    const bool all_heads = (y % hblks) * 4 + 3 < G;
+    const int n_steady = (EVEN && all_heads) ? max(min(seen_whole, kb1 - kb0 - 4), 0) & ~1 : 0;
+    int it = 0;
+    if (a.near) {
+      for (; it < n_steady; it += 2) {
+        steady(kst[0], vst[0], kps[0], vps[0], kst[1], vst[1], kps[1], vps[1], it, std::true_type{});
+        steady(kst[1], vst[1], kps[1], vps[1], kst[0], vst[0], kps[0], vps[0], it + 1, std::true_type{});
+      }
+    } else {
+      for (; it < n_steady; it += 2) {
+        steady(kst[0], vst[0], kps[0], vps[0], kst[1], vst[1], kps[1], vps[1], it, std::false_type{});
+        steady(kst[1], vst[1], kps[1], vps[1], kst[0], vst[0], kps[0], vps[0], it + 1, std::false_type{});
+      }
+    }
+    for (; it < seen_whole; it += 2) {
+      round(kst[0], vst[0], kps[0], vps[0], kst[1], vst[1], kps[1], vps[1], it, std::true_type{});
+      round(kst[1], vst[1], kps[1], vps[1], kst[0], vst[0], kps[0], vps[0], it + 1, std::true_type{});
+    }
+    for (; it < steps; it += 2) {
+      round(kst[0], vst[0], kps[0], vps[0], kst[1], vst[1], kps[1], vps[1], it, std::false_type{});
+      if (it + 1 < steps) round(kst[1], vst[1], kps[1], vps[1], kst[0], vst[0], kps[0], vps[0], it + 1, std::false_type{});
     }
 
     // The second set hands its sums to the first, lane by lane (both hold the same columns and channels):
@@ -778,8 +932,7 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
 
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      lsum[u] += __shfl_xor(lsum[u], 16, 64);
-      lsum[u] += __shfl_xor(lsum[u], 32, 64);
+      // (lsum[u] is the column's whole sum in every lane of the column: the matrix instruction added over all keys)
       if (!col_ok[u]) continue;
       // o[u][dt][j] is channel 16 dt + 4 g + j of column c
       if (a.splits == 1) {
@@ -868,7 +1021,7 @@ extern "C" int ns_attn_mfma_page_size() { return PS; }
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
-                            int coop, hipStream_t stream) {
+                            int coop, long pool_pages, hipStream_t stream) {
   if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size != PS || window < 0 ||
       splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
     return NS_ERR_BAD_ARG;
@@ -883,6 +1036,8 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   a.tiles = tiles; a.block_table = block_table;
   a.q_stride = q_stride; a.table_stride = table_stride; a.n_tiles = n_tiles; a.heads = heads; a.kv_heads = kv_heads;
   a.hp = hp; a.splits = splits; a.window = window;
+  const long page_bytes = (long)kv_heads * HD * PS * 2;
+  a.near = pool_pages > 0 && pool_pages < (1L << 24) && page_bytes < (1L << 24) && pool_pages * page_bytes <= (1L << 32);
   a.scale_log2 = scale * 1.4426950408889634f;
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);

@@ -662,7 +662,8 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     lib = build.attn(head_dim, page)
     _check(lib.ns_attn_mfma(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tiles),
                             _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads),
-                            c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_int(1 if coop else 0), _stream()),
+                            c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_int(1 if coop else 0),
+                            ctypes.c_long(k_cache.shape[0]), _stream()),
            "attention_mfma")
     return out
 
