@@ -22,6 +22,12 @@
 // Query at position p sees keys max(0, p - window + 1) .. p.  Scores, soft-max and sums are 32-bit.
 // With splits > 1 the keys of a tile are cut into `splits` contiguous ranges of whole 32-key blocks;
 // each range writes its un-normalised output, maximum and sum, and a second small kernel joins them.
+//
+// Three kernels: attn_mfma_kernel (a wave per tile, or a workgroup per tile for decode rows), attn_prefill_kernel
+// (prompt portions in tiles of 32 tokens, four heads of a group share each block of keys through LDS) and, for head
+// sizes 64 and 128 and pages of 8 tokens or more, attn_prefill32_kernel in attn_prefill32.h (the same sharing on the
+// 32x32 matrix instruction with keys and values loaded straight into LDS).  Compiled with -DNS_PREFILL16 the second
+// serves those head sizes too: that is for measurements of one against the other.
 #include "common.h"
 #include <type_traits>
 
@@ -957,6 +963,8 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
   }
 }
 
+#include "attn_prefill32.h"
+
 // Joining the key ranges: out[col] = sum_s o_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*), m* = max_s m_s.
 // One wave per (tile, token of the tile, head); lane s first holds range s (at most 64 ranges), so the maxima and
 // weights are formed by wave reductions, then the lanes split the channels and add the ranges in order.  The ranges'
@@ -1046,6 +1054,14 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (qt == 2 && SHARED_OK) {
     const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
+#ifndef NS_PREFILL16
+    if (DMA_OK) {
+      if (coop)
+        attn_prefill32_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>(a);
+      else
+        attn_prefill32_kernel<2><<<(unsigned)wgs, 512, 0, stream>>>(a);
+    } else
+#endif
     if (coop)
       attn_prefill_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>(a);
     else

@@ -630,14 +630,17 @@ TILE_INTS = 8  # ints per attention tile descriptor: request, first token, first
 
 def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_heads: int, head_dim: int, scale: float,
                    window: int = 0, hp: int = 1, splits: int = 1,
-                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1, coop: bool = False) -> torch.Tensor:
+                   workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1, coop: bool = False,
+                   short_offsets: bool = True) -> torch.Tensor:
     """bfloat16 attention on the matrix cores for the tiles described in ``tiles`` (int32 [n_tiles, 8]: request, first
     token of the tile among the request's tokens of this step, row of the request's first token in ``q``, tokens of the
     request in this step, keys after this step, three zeros).  ``hp`` heads of a group times 16/hp tokens make a tile;
     with ``qt`` = 2 (only with hp = 1) a tile is 32 tokens.  ``splits`` > 1 cuts the keys of every tile
     into that many ranges (at most 64) and needs ``workspace`` = (part_o, part_ml) float32 tensors.  With ``coop`` the four
     waves of a workgroup share each tile and range (for decode, where a wave's chain of loads is what takes the time); with
-    ``qt`` = 2 it asks for workgroups of one set of four waves instead of two (for long rows of keys)."""
+    ``qt`` = 2 it asks for workgroups of one set of four waves instead of two (for long rows of keys).  A pool within
+    4 GiB is addressed with 32-bit offsets from its start; ``short_offsets`` = False keeps every address 64 bits wide
+    whatever the pool's size (the form that larger pools take)."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
     if not mfma_attention_takes(q.dtype, head_dim, page):
         raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
@@ -663,7 +666,7 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     _check(lib.ns_attn_mfma(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tiles),
                             _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads),
                             c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_int(1 if coop else 0),
-                            ctypes.c_long(k_cache.shape[0]), _stream()),
+                            ctypes.c_long(k_cache.shape[0] if short_offsets else 0), _stream()),
            "attention_mfma")
     return out
 

@@ -582,7 +582,7 @@ def test_untile_gives_the_matrix_back(n, k):
 
 
 def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0,
-              chunk_splits=1):
+              chunk_splits=1, short_offsets=True):
     n = sum(lens)
     indptr = [0]
     for l in lens:
@@ -601,7 +601,8 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
         if chunk_splits > 1:  # filled with NaN: a range that is read without having been written shows
             ws = (torch.full((cols * chunk_splits * hd,), float("nan"), device=DEV), torch.full((cols * chunk_splits * 2,), float("nan"), device=DEV))
         ops.attention_mfma(q, out, k, v, i32(ct), table.to(DEV), heads, kvh, hd, 1 / math.sqrt(hd), window=window, hp=1,
-                           splits=chunk_splits, workspace=ws, qt=qt, coop=coop and qt == 2)  # coop: one set of waves per workgroup
+                           splits=chunk_splits, workspace=ws, qt=qt, coop=coop and qt == 2,  # coop: one set of waves per workgroup
+                           short_offsets=short_offsets)
     if dt:
         hp = 1
         while hp < min(group, 16):
@@ -639,6 +640,63 @@ def test_attention_mfma(case, heads, kvh, hd, page):
         assert u <= 4, f"{case} splits={splits} qt={qt} coop={coop} chunk_splits={chunk_splits}: {u:.2f} ulps"
 
 
+# The prompt kernel for head sizes 64 and 128 brings keys and values straight into LDS, a page id per page of a block of
+# 32 keys: every page size it takes (four, two, one page a block, a block inside a page), a group of three heads (a wave
+# of the workgroup has no head), a group of eight (two workgroups a key/value head), and addresses of 64 bits.
+@pytest.mark.parametrize("case", ["prefill", "mixed", "long", "beyond64pages", "far"])
+@pytest.mark.parametrize("heads,kvh,hd,page,short_offsets", [(8, 2, 128, 8, True), (8, 2, 128, 32, True), (16, 4, 64, 64, True), (4, 1, 64, 8, False),
+                                                             (6, 2, 128, 16, True), (8, 1, 128, 16, False), (4, 2, 64, 128, False)])
+def test_attention_mfma_prompt_kernel_page_sizes_and_groups(case, heads, kvh, hd, page, short_offsets):
+    ops = _ops()
+    starts, lens = CASES[case]
+    torch.manual_seed(14)
+    total = [s + l for s, l in zip(starts, lens)]
+    pages = sum(-(-t // page) for t in total) + 3
+    table = scattered_tables(total, page, pages, seed=3)
+    k, v = make_cache(pages, page, kvh, hd, torch.bfloat16)
+    kvs = fill_cache(k, v, table, total, page, kvh, hd, torch.bfloat16, seed=4)
+    n = sum(lens)
+    q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
+    ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
+    for coop, chunk_splits in ((False, 1), (True, 1), (True, 3), (False, 16)):
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, qt=2, coop=coop, chunk_splits=chunk_splits, short_offsets=short_offsets)
+        u = ulps_of_row_max(out.cpu(), ref).max()
+        assert u <= 4, f"{case} coop={coop} chunk_splits={chunk_splits}: {u:.2f} ulps"
+
+
+@pytest.mark.parametrize("hd,page", [(128, 16), (64, 8), (128, 32)])
+@pytest.mark.parametrize("coop", [False, True])
+def test_attention_prompt_dominant_key_at_block_and_ring_edges(hd, page, coop):
+    """A prompt portion of 70 tokens over some hundred keys; one key is made to dominate every query that sees it, so
+    their outputs must be its value.  Done for keys around the edges of the kernel's blocks of 32 keys, of its ring of
+    three buffers (96 keys), of the pages, of the halves that two sets of waves take, and inside the portion itself, where
+    only later tokens see the key."""
+    ops = _ops()
+    heads, kvh = 8, 2
+    n, total, dtype = 70, 430, torch.bfloat16
+    start = total - n
+    pages = -(-total // page) + 2
+    table = scattered_tables([total], page, pages, seed=6)
+    torch.manual_seed(9)
+    base = torch.randn(heads * hd, dtype=dtype, device=DEV)
+    q = base.repeat(n, 1).contiguous()  # every token asks the same
+    for special in (0, 1, 31, 32, 33, 63, 64, 95, 96, 97, 127, 128, 191, 192, 193, 215, 216, 287, 288, 359, 360, 361, 383, 384, 400, 428, 429):
+        k, v = make_cache(pages, page, kvh, hd, dtype)
+        kvs = fill_cache(k, v, table, [total], page, kvh, hd, dtype, seed=special, scale=0.05)
+        pg, off = int(table[0, special // page]), special % page
+        for h in range(kvh):
+            k[pg, h, off] = (base.view(heads, hd)[h * (heads // kvh)] * 4).to(dtype)  # aligned with the group's first query head
+        kvs[0][0][special] = k[pg, :, off].cpu()
+        out = _run_mfma(ops, q, k, v, table, [start], [n], heads, kvh, hd, qt=2, coop=coop).view(n, heads, hd).float().cpu()
+        ref = plain_paged_attention(q.view(n, heads, hd), kvs, [start], [n], heads).reshape(n, -1)
+        assert ulps_of_row_max(out.reshape(n, -1), ref).max() <= 4, f"key {special}"
+        for h in range(kvh):
+            want = kvs[0][1][special, h].float()
+            for t in range(n):
+                if start + t >= special:
+                    assert torch.allclose(out[t, h * (heads // kvh)], want, atol=0.05), f"key {special}, token {t}: output is not its value"
+
+
 @pytest.mark.parametrize("kernel", ["generic", "mfma"])
 def test_attention_far_key_and_page_edges(kernel):
     """One key among hundreds is made to dominate: its score stands out, so the output must be its value.
@@ -670,9 +728,10 @@ def test_attention_far_key_and_page_edges(kernel):
 
 @pytest.mark.parametrize("kernel", ["generic", "mfma"])
 @pytest.mark.parametrize("window", [5, 16, 40])
-def test_attention_window(kernel, window):
+@pytest.mark.parametrize("hd,page", [(32, 8), (128, 16), (64, 8)])  # (the prompt kernels: one for head sizes 64 and 128, one for the others)
+def test_attention_window(kernel, window, hd, page):
     ops = _ops()
-    heads, kvh, hd, page = 4, 2, 32, 8
+    heads, kvh = 4, 2
     starts, lens = [50, 0, 100], [1, 45, 20]
     dtype = torch.bfloat16
     total = [s + l for s, l in zip(starts, lens)]
