@@ -1055,7 +1055,15 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
     const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
 #ifndef NS_PREFILL16
-    if (DMA_OK) {
+    // attn_prefill32_kernel counts its loads by hand, so it must have no others: were it ever compiled with registers
+    // spilled to scratch memory (whose accesses count among the loads), the other kernel takes its place.
+    static const bool counts_hold = [] {
+      hipFuncAttributes one, two;
+      return hipFuncGetAttributes(&one, reinterpret_cast<const void*>(&attn_prefill32_kernel<1>)) == hipSuccess &&
+             hipFuncGetAttributes(&two, reinterpret_cast<const void*>(&attn_prefill32_kernel<2>)) == hipSuccess && one.localSizeBytes == 0 &&
+             two.localSizeBytes == 0;
+    }();
+    if (DMA_OK && counts_hold) {
       if (coop)
         attn_prefill32_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>(a);
       else

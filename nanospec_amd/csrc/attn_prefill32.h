@@ -43,9 +43,6 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 
-#ifndef NS_VALU_PER_MFMA32
-#define NS_VALU_PER_MFMA32 7
-#endif
 constexpr bool DMA_OK = (HD == 64 || HD == 128) && PS >= 8;  // (other sizes: attn_prefill_kernel)
 constexpr int QS = HD / 16;                // matrix instructions per block for the scores
 constexpr int CT = HD / 32 > 0 ? HD / 32 : 1;                // tiles of 32 channels of the output
@@ -63,17 +60,6 @@ __device__ __forceinline__ float max_with_other_half(float x) {  // over lanes l
   const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   return fmaxf(__uint_as_float(h[0]), __uint_as_float(h[1]));
 }
-
-// In a stretch of straight code: two LDS reads ahead, then N times one matrix instruction, the LDS read of the one after
-// next and V vector instructions, in that order of issue (a matrix instruction waits for its operand; with the read
-// issued two instructions earlier the wait is short and the vector instructions do not stand behind it).
-#define NS_STAGE_LDS(N, V)                                    \
-  __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);          \
-  _Pragma("unroll") for (int sg_ = 0; sg_ < (N); ++sg_) {     \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        \
-    __builtin_amdgcn_sched_group_barrier(0x002, (V), 0);      \
-  }
 
 // Wait until at most `n` of this wave's loads are still on their way (and for nothing else).
 #define NS_WAIT_LOADS(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
@@ -185,10 +171,15 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
 #pragma unroll
       for (int p = 0; p < PPB; ++p) ids[p] = stable[min(max(first + p, lo_slot), hi_slot)];
     };
-    auto pick = [&](const auto(&per_page)[PPB], int slot) {
+    auto pick = [&](const auto(&per_page)[PPB], int slot) {  // per_page[slot], with per_page in scalar registers
       auto x = per_page[0];
 #pragma unroll
-      for (int p = 1; p < PPB; ++p) x = slot == p ? per_page[p] : x;
+      for (int p = 1; p < PPB; ++p) {
+        x = slot == p ? per_page[p] : x;
+        // (kept a chain of selects: rewritten as an array indexed by the lane's slot, the ids would move to scratch
+        // memory, whose accesses count among the loads that the rounds' waits count)
+        if (PPB > 2) asm volatile("" : "+v"(x));
+      }
       return x;
     };
     typedef __attribute__((address_space(3))) void* lds_ptr;
