@@ -1026,6 +1026,25 @@ extern "C" int ns_attn_mfma_page_size() { return PS; }
 
 // Workspace, when splits > 1: with T = qt*16/hp tokens in a tile, part_o holds n_tiles*T*heads*splits*HD floats and
 // part_ml n_tiles*T*heads*splits*2.
+// Which kernel takes prompt portions in tiles of 32 tokens in this library: 32 attn_prefill32_kernel, 16
+// attn_prefill_kernel, 0 attn_mfma_kernel.  attn_prefill32_kernel counts its loads by hand, so it must have no others:
+// were it ever compiled with registers spilled to scratch memory (whose accesses count among the loads), the 16x16
+// kernel takes its place.
+static int prompt_form() {
+  if (!SHARED_OK) return 0;
+#ifndef NS_PREFILL16
+  static const bool counts_hold = [] {
+    hipFuncAttributes one, two;
+    return hipFuncGetAttributes(&one, reinterpret_cast<const void*>(&attn_prefill32_kernel<1>)) == hipSuccess &&
+           hipFuncGetAttributes(&two, reinterpret_cast<const void*>(&attn_prefill32_kernel<2>)) == hipSuccess && one.localSizeBytes == 0 &&
+           two.localSizeBytes == 0;
+  }();
+  if (DMA_OK && counts_hold) return 32;
+#endif
+  return 16;
+}
+extern "C" int ns_attn_prompt_form(void) { return prompt_form(); }
+
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
@@ -1055,15 +1074,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
     const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
 #ifndef NS_PREFILL16
-    // attn_prefill32_kernel counts its loads by hand, so it must have no others: were it ever compiled with registers
-    // spilled to scratch memory (whose accesses count among the loads), the other kernel takes its place.
-    static const bool counts_hold = [] {
-      hipFuncAttributes one, two;
-      return hipFuncGetAttributes(&one, reinterpret_cast<const void*>(&attn_prefill32_kernel<1>)) == hipSuccess &&
-             hipFuncGetAttributes(&two, reinterpret_cast<const void*>(&attn_prefill32_kernel<2>)) == hipSuccess && one.localSizeBytes == 0 &&
-             two.localSizeBytes == 0;
-    }();
-    if (DMA_OK && counts_hold) {
+    if (prompt_form() == 32) {
       if (coop)
         attn_prefill32_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>(a);
       else

@@ -671,6 +671,13 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     return out
 
 
+def attention_prompt_form(head_dim: int, page_size: int) -> int:
+    """Which kernel of the library for this head and page size takes prompt portions in tiles of 32 tokens: 32 the one
+    on the 32x32 matrix instruction with loads straight into LDS, 16 the one on the 16x16 instruction with keys shared
+    through LDS, 0 the one without sharing."""
+    return int(build.attn(head_dim, page_size).ns_attn_prompt_form())
+
+
 # ------------------------------------------------------------------------------------------------ sampling
 
 

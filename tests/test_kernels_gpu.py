@@ -664,6 +664,17 @@ def test_attention_mfma_prompt_kernel_page_sizes_and_groups(case, heads, kvh, hd
         assert u <= 4, f"{case} coop={coop} chunk_splits={chunk_splits}: {u:.2f} ulps"
 
 
+def test_attention_prompt_kernel_in_use():
+    """Head sizes 64 and 128 with pages of 8 tokens or more run the 32x32 prompt kernel (it steps aside if it was ever
+    compiled with scratch memory: then this fails, and says that the tests above did not run it), the other sizes
+    the kernels they are made for."""
+    ops = _ops()
+    for hd, page in ((64, 8), (64, 16), (64, 64), (64, 128), (128, 8), (128, 16), (128, 32)):
+        assert ops.attention_prompt_form(hd, page) == 32, (hd, page)
+    assert ops.attention_prompt_form(32, 16) == 16 and ops.attention_prompt_form(96, 16) == 16
+    assert ops.attention_prompt_form(48, 4) == 0 and ops.attention_prompt_form(144, 16) == 0
+
+
 @pytest.mark.parametrize("hd,page", [(128, 16), (64, 8), (128, 32)])
 @pytest.mark.parametrize("coop", [False, True])
 def test_attention_prompt_dominant_key_at_block_and_ring_edges(hd, page, coop):
