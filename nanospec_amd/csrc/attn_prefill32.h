@@ -267,9 +267,15 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       }
       if (nb > 2) load_k(ids_v, kb0 + 2, 2);
     }
-    NS_WAIT_LOADS(0);
+    // (loads land in the order they were asked for: the first scores wait for the keys of block 0 only, round 0 for the
+    // values of block 0 and the keys of block 1; a range of fewer than three blocks waits for all it asked for)
+    if (kb1 - kb0 > 2)
+      NS_WAIT_LOADS(4 * IPW);
+    else
+      NS_WAIT_LOADS(0);
     __builtin_amdgcn_s_barrier();
     if (head_ok && kb0 < kb1) scores(0);
+    if (kb1 - kb0 > 2) NS_WAIT_LOADS(2 * IPW);
     __builtin_amdgcn_s_barrier();  // (the scores' LDS reads are done: a matrix instruction has taken each of them)
 
     // What round `it` asks for: the keys of block it + 3 over those of block it, whose scores are formed, and the values
