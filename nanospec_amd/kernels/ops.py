@@ -418,26 +418,66 @@ def linear_resid_norm(x: torch.Tensor, w: TiledWeight, resid: torch.Tensor, next
     return PreNormed(x_next, ssq, w.n, eps)
 
 
+def _wide_cost(tiles: int, per_group: int, ksplit: int, k_tiles: int, units: int) -> int:
+    """What the busiest compute unit streams, in row tiles times k tiles: a product of few rows takes as long as that."""
+    groups = -(-tiles // per_group)
+    return -(-groups * ksplit // units) * per_group * -(-k_tiles // ksplit)
+
+
 def wide_plan(n: int, k: int, rows: int = SKINNY_MAX_ROWS, units: int | None = None) -> tuple[int, int]:
     """(ranges K is cut into, 16-row tiles per wave) of ``linear_wide``: two tiles per wave when there are rows enough
     (and at most 64 rows of x), then as many ranges as give every compute unit about one workgroup, with at least four k
     tiles of 128 per range (more, shorter ranges were measured slower once the kernel that joins them is counted: 37 against
-    31 us for the down-projection of the 8B shape at 64 rows with 10 and with 4 ranges).  ``units``: the GPU's compute
-    units (the current device's by default)."""
+    31 us for the down-projection of the 8B shape at 64 rows with 10 and with 4 ranges).  With one tile per wave and up to
+    64 rows a workgroup may have three waves instead of four (``wide_waves``); the ranges are chosen for whichever of the
+    two leaves the busiest compute unit the least to stream.  ``units``: the GPU's compute units (the current device's by
+    default)."""
     units = units or compute_units(torch.cuda.current_device())
     nt = 2 if n >= 8192 and rows <= SKINNY_MAX_ROWS else 1
-    row_groups = -(-n // (64 * nt))
     k_tiles = -(-k // 128)
-    return max(1, min(16, k_tiles // 4, round(units / row_groups))), nt
+    most = max(1, min(16, k_tiles // 4))
+    ranges = lambda per_group: max(1, min(most, round(units / -(-n // (16 * per_group)))))
+    if nt != 1 or rows > SKINNY_MAX_ROWS:
+        return ranges(4 * nt), nt
+    tiles = -(-n // 16)
+    four, three = ranges(4), ranges(3)
+    return (three if _wide_cost(tiles, 3, three, k_tiles, units) < _wide_cost(tiles, 4, four, k_tiles, units) else four), nt
 
 
-def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
-                out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0, defer: bool = False):
+def wide_waves(n: int, k: int, rows: int, ksplit: int, nt: int, gated: bool = False, units: int | None = None) -> tuple[int, bool]:
+    """(waves per workgroup, by half tiles) of ``linear_wide`` for a product cut as given: what deals the row tiles most
+    evenly to the compute units.  One matrix, one tile per wave, up to 64 rows: three waves instead of four where that
+    leaves the busiest unit less.  Gate and up in one range: four waves of a whole tile of each (8 half tiles a workgroup),
+    seven or four waves of half a tile of each (7 or 4 a workgroup); at the 8B shape 1,792 half tiles are 7 for each of 256
+    units instead of 8 for each of 224 (42 against 51 us at 64 rows; the 1B shape's 1,024 as 4 for each: 17 against 25 us)."""
+    units = units or compute_units(torch.cuda.current_device())
+    if rows > SKINNY_MAX_ROWS or nt != 1:
+        return 4, False
+    tiles, k_tiles = -(-n // 16), -(-k // 128)
+    if gated:
+        if ksplit != 1 or -(-tiles // 4) >= units:  # (whole tiles fill the GPU: measured level or ahead, 163 against 166 us at the 70B shape)
+            return 4, False
+        options = [(-(-(-(-tiles // 4)) // units) * 8, 4, False), (-(-(-(-2 * tiles // 7)) // units) * 7, 7, True),
+                   (-(-(-(-2 * tiles // 4)) // units) * 4, 4, True)]
+        _, waves, halves = min(options, key=lambda o: o[0])  # (the first of equals: the fewest workgroups, each reads x)
+        return waves, halves
+    three = _wide_cost(tiles, 3, ksplit, k_tiles, units) < _wide_cost(tiles, 4, ksplit, k_tiles, units)
+    return (3 if three else 4), False
+
+
+def linear_wide(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
+                out_f32: bool = False, workspace: torch.Tensor | None = None, ksplit: int = 0, nt: int = 0, defer: bool = False,
+                waves: int = 0, halves: bool | None = None):
     """bfloat16 x @ w.T for up to 64 rows from a tiled weight (up to 128 with ``nt=1`` and no ``w2``), with the tile of x
     shared through LDS by the four waves of
     a workgroup and K cut into ``ksplit`` ranges that a second kernel adds up; with ``w2``: silu(x @ w.T) * (x @ w2.T).
     ``workspace``: float32, (2 if w2 else 1) * ksplit * rows * w.n values (none for a single range).  ``defer`` (not with
-    ``w2``): with more than one range the second kernel is left out and a ``PartialSums`` over the workspace comes back."""
+    ``w2``): with more than one range the second kernel is left out and a ``PartialSums`` over the workspace comes back.
+    ``waves``, ``halves``: waves per workgroup and whether gate and up go by half tiles (``wide_waves`` by default).
+    ``x`` may be a ``PreNormed`` (at most 16 rows, one range)."""
+    pre = x if isinstance(x, PreNormed) else None
+    if pre is not None:
+        x = pre.x
     _gpu(x, out, workspace)
     if x.dim() != 2 or x.shape[1] != w.k or not tiled_takes(x, w.k, WIDE_TALL_ROWS):
         raise KernelRefused(f"linear_wide takes bfloat16 x [rows <= {WIDE_TALL_ROWS}, {w.k}] with an inner size that is a "
@@ -460,10 +500,21 @@ def linear_wide(x: torch.Tensor, w: TiledWeight, w2: TiledWeight | None = None, 
         workspace = torch.empty(need, dtype=torch.float32, device=x.device)
     if need and (workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous()):
         raise KernelRefused("linear_wide: workspace too small")
-    _check(build.core().ns_gemm_wide_bf16(_ptr(None if defer else out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data),
-                                          _ptr(w2.data if w2 is not None else None), c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)),
-                                          c_int(w.n if defer else out.stride(0)), c_int(1 if w2 is not None else 0),
-                                          c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), c_int(1 if defer else 0), _stream()),
+    if not waves:
+        waves, dealt_halves = wide_waves(w.n, w.k, m, ksplit, nt, gated=w2 is not None)
+        halves = dealt_halves if halves is None else halves
+    halves = bool(halves)
+    if pre is not None and (ksplit != 1 or defer):
+        raise KernelRefused("linear_wide: a pre-normed input goes with one range of K")
+    if halves and (w2 is None or ksplit != 1 or nt != 1 or m > SKINNY_MAX_ROWS or waves not in (4, 7)):
+        raise KernelRefused("linear_wide: half tiles go with two matrices, one range, one tile per wave, up to 64 rows, 4 or 7 waves")
+    if not halves and waves != 4 and not (waves == 3 and w2 is None and nt == 1 and m <= SKINNY_MAX_ROWS):
+        raise KernelRefused("linear_wide: workgroups of 4 waves, or of 3 for one matrix with one tile per wave and up to 64 rows")
+    _check(build.core().ns_gemm_wide_dealt_bf16(_ptr(None if defer else out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data),
+                                                _ptr(w2.data if w2 is not None else None), c_int(m), c_int(w.n), c_int(w.k), c_int(x.stride(0)),
+                                                c_int(w.n if defer else out.stride(0)), c_int(1 if w2 is not None else 0),
+                                                c_int(1 if out_f32 else 0), c_int(ksplit), c_int(nt), c_int(1 if defer else 0),
+                                                c_int(waves), c_int(1 if halves else 0), *_prenorm_args(pre, m, "linear_wide"), _stream()),
            "linear_wide")
     return PartialSums(workspace, ksplit, m, w.n, x.dtype) if defer else out
 

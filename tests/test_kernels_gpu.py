@@ -150,6 +150,58 @@ def test_linear_wide(m, n, k):
         assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0
 
 
+@pytest.mark.parametrize("m", [17, 33, 48, 64, 5])
+@pytest.mark.parametrize("n,k", [(48, 64), (130, 200), (1000, 4096), (257, 1064), (1440, 512)])
+def test_linear_wide_dealt_to_the_compute_units(m, n, k):
+    """The same kernel with three waves a workgroup (one matrix) and with gate and up by half tiles in workgroups of four
+    or seven waves: every form adds a sum's terms in the same order, so the results are equal bit for bit."""
+    ops = _ops()
+    from nanospec_amd.kernels import KernelRefused
+
+    torch.manual_seed(m + n + k + 1)
+    x = torch.randn(m + 3, k + 8, dtype=torch.bfloat16, device=DEV)[:m, :k]
+    w = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    wt, wt2 = ops.TiledWeight(w), ops.TiledWeight(w2)
+    ref = x.cpu().float() @ w.cpu().float().T
+    k_tiles = -(-k // 128)
+    for ks in sorted({1, 2, min(3, k_tiles)}):
+        if ks > k_tiles:
+            continue
+        four = ops.linear_wide(x, wt, out_f32=True, ksplit=ks, nt=1, waves=4)
+        three = ops.linear_wide(x, wt, out_f32=True, ksplit=ks, nt=1, waves=3)
+        torch.testing.assert_close(three.cpu(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(k))
+        assert torch.equal(three, four), f"{ks} ranges"
+        if ks > 1:
+            part = ops.linear_wide(x, wt, ksplit=ks, nt=1, waves=3, defer=True)
+            assert torch.equal(ops.reduce_partial(part), ops.linear_wide(x, wt, ksplit=ks, nt=1, waves=4))
+    u = x.cpu().float() @ w2.cpu().float().T
+    whole = ops.linear_wide(x, wt, w2=wt2, ksplit=1, nt=1, waves=4, halves=False)
+    assert ulps_of_row_max(whole.cpu(), ref * torch.sigmoid(ref) * u).max() <= 1.0
+    for waves in (4, 7):
+        halves = ops.linear_wide(x, wt, w2=wt2, ksplit=1, nt=1, waves=waves, halves=True)
+        assert torch.equal(halves, whole), f"half tiles, {waves} waves"
+    assert torch.equal(ops.linear_wide(x, wt, w2=wt2, ksplit=1, nt=1), whole)  # whichever form the plan deals
+    for bad in (dict(waves=7), dict(waves=3, w2=wt2), dict(waves=7, halves=True), dict(w2=wt2, waves=4, halves=True, ksplit=2),
+                dict(waves=3, nt=2), dict(waves=5)):
+        with pytest.raises(KernelRefused):
+            ops.linear_wide(x, wt, **{"ksplit": 1, "nt": 1, **bad})
+
+
+def test_wide_plans_deal_evenly():
+    """What the plans choose at the three shapes' sizes on 256 compute units: q/k/v of the 8B shape in workgroups of three
+    waves over two ranges (256 workgroups where four waves over three ranges are 288), gate and up by half tiles."""
+    ops = _ops()
+    assert ops.wide_plan(6144, 4096, 64, units=256) == (2, 1) and ops.wide_waves(6144, 4096, 64, 2, 1, units=256) == (3, False)
+    assert ops.wide_plan(4096, 4096, 64, units=256) == (4, 1) and ops.wide_waves(4096, 4096, 64, 4, 1, units=256) == (4, False)
+    assert ops.wide_plan(4096, 14336, 64, units=256) == (4, 1) and ops.wide_waves(4096, 14336, 64, 4, 1, units=256) == (4, False)
+    assert ops.wide_waves(14336, 4096, 64, 1, 1, gated=True, units=256) == (7, True)   # 1,792 half tiles: 7 for each of 256 units
+    assert ops.wide_waves(8192, 2048, 64, 1, 1, gated=True, units=256) == (4, True)    # 1,024 half tiles: 4 for each
+    assert ops.wide_waves(28672, 8192, 64, 1, 1, gated=True, units=256) == (4, False)  # 448 workgroups of whole tiles fill the GPU
+    assert ops.wide_waves(14336, 4096, 100, 1, 1, units=256) == (4, False)             # more than 64 rows: four waves
+    assert ops.wide_waves(14336, 4096, 64, 2, 1, gated=True, units=256) == (4, False)  # gate and up over ranges: whole tiles
+
+
 def test_linear_tiled_refuses():
     ops = _ops()
     from nanospec_amd.kernels import KernelRefused
@@ -371,6 +423,19 @@ def test_product_that_updates_the_residual_and_feeds_the_next_norm(m, hidden, in
     up = normed.float() @ w4.float().T
     act = ops.linear_tiled(pre, ops.TiledWeight(w3.to(DEV)), w2=ops.TiledWeight(w4.to(DEV)))
     assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * up).max() <= 2.0
+    # the kernel that shares x through LDS takes the same input: whole tiles, half tiles in workgroups of 4 and 7 waves,
+    # one matrix in workgroups of 3 and 4 waves
+    t3, t4 = ops.TiledWeight(w3.to(DEV)), ops.TiledWeight(w4.to(DEV))
+    for waves, halves in ((4, False), (4, True), (7, True)):
+        act = ops.linear_wide(pre, t3, w2=t4, ksplit=1, nt=1, waves=waves, halves=halves)
+        assert ulps_of_row_max(act.cpu(), ref * torch.sigmoid(ref) * up).max() <= 2.0, (waves, halves)
+    for waves in (3, 4):
+        assert ulps_of_row_max(ops.linear_wide(pre, t3, ksplit=1, nt=1, waves=waves, out_f32=True).cpu(), ref).max() <= 1.0
+    if hidden >= 256:
+        from nanospec_amd.kernels import KernelRefused
+
+        with pytest.raises(KernelRefused):
+            ops.linear_wide(pre, t3, ksplit=2, nt=1)  # a pre-normed input goes with one range
 
 
 @pytest.mark.parametrize("m", [65, 81, 100, 113, 128])
