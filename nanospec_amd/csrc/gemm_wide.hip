@@ -317,12 +317,21 @@ static int launch_wide(float* partial, const bf16_t* x, const bf16_t* wt, const 
   return ns_launch_status();
 }
 
-// 65 to 128 rows: one matrix, one row tile per wave (the x tile takes 72 KiB of LDS at 128 rows).
+// 65 to 128 rows: one matrix, one row tile per wave (the x tile takes 72 KiB of LDS at 128 rows), or gate and up by half
+// tiles, which need one set of sums where whole tiles of both need two.
 template <int MT>
-static int launch_wide_tall(float* partial, const bf16_t* x, const bf16_t* wt, int M, int N, int K, int x_stride, int ksplit,
-                            void* direct_out, int out_stride, int out_f32, hipStream_t stream) {
+static int launch_wide_tall(float* partial, const bf16_t* x, const bf16_t* wt, const bf16_t* wt2, int M, int N, int K, int x_stride,
+                            int ksplit, int waves, int halves, void* direct_out, int out_stride, int out_f32, hipStream_t stream) {
   const WideNorm nl;
   const int row_tiles = (N + 15) / 16;
+  if (halves) {  // (checked by the caller: two matrices, one range of K, 4 or 7 waves)
+    const int units = 2 * row_tiles;
+    if (waves == 7)
+      gemm_wide_kernel<MT, 1, 1, 7, true><<<dim3((units + 6) / 7, 1), 448, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, 1, direct_out, out_stride, out_f32, 0, 0, nl);
+    else
+      gemm_wide_kernel<MT, 1, 1, 4, true><<<dim3((units + 3) / 4, 1), 256, 0, stream>>>(partial, x, wt, wt2, M, N, K, x_stride, 1, direct_out, out_stride, out_f32, 0, 0, nl);
+    return ns_launch_status();
+  }
   dim3 grid((row_tiles + 3) / 4, ksplit);
   gemm_wide_kernel<MT, 1, 1><<<grid, 256, 0, stream>>>(partial, x, wt, nullptr, M, N, K, x_stride, ksplit, direct_out, out_stride, out_f32, 0, 0, nl);
   return ns_launch_status();
@@ -332,16 +341,16 @@ static int launch_wide_tall(float* partial, const bf16_t* x, const bf16_t* wt, i
 // defer (with ksplit > 1 and epi 0): the ranges stay in the workspace as [ksplit][M][N] and nothing is written to out; they
 // are added later by ns_wide_reduce or by a norm that reads them (ns_rmsnorm_partial).
 // waves: waves per workgroup, 4, or 3 (one matrix, nt 1, up to 64 rows), or 7 (with halves).  halves: gate and up by half row
-// tiles (epi 1, one range of K, nt 1, up to 64 rows, 4 or 7 waves).
+// tiles (epi 1, one range of K, nt 1, 4 or 7 waves; also for 65 to 128 rows).
 static int wide_product(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N, int K,
                         int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer, int waves, int halves,
                         WideNorm nl, hipStream_t stream) {
   if (nl.ssq_in && (M > 16 || ksplit != 1 || nl.parts_in <= 0)) return NS_ERR_BAD_ARG;
-  if (halves ? (epi != 1 || ksplit != 1 || nt != 1 || M > 64 || (waves != 4 && waves != 7))
+  if (halves ? (epi != 1 || ksplit != 1 || nt != 1 || (waves != 4 && waves != 7))
              : (waves != 4 && !(waves == 3 && epi == 0 && nt == 1 && M <= 64)))
     return NS_ERR_BAD_ARG;
   if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K & 7) || (x_stride & 7) || x_stride < K || out_stride < N) return NS_ERR_BAD_ARG;
-  if (M > 64 && (wt2 != nullptr || nt != 1)) return NS_ERR_BAD_ARG;  // 65 to 128 rows: one matrix, one row tile per wave
+  if (M > 64 && ((wt2 != nullptr && !halves) || nt != 1)) return NS_ERR_BAD_ARG;  // 65 to 128 rows: one row tile per wave; two matrices by half tiles only
   if ((epi == 1) != (wt2 != nullptr) || (epi != 0 && epi != 1) || (epi == 1 && out_f32)) return NS_ERR_BAD_ARG;
   const int KT = (K + 127) / 128;
   if (ksplit < 1 || ksplit > KT || ksplit > 65535 || (nt != 1 && nt != 2) || (ksplit > 1 && !workspace)) return NS_ERR_BAD_ARG;
@@ -354,10 +363,10 @@ static int wide_product(void* out, void* workspace, const void* x, const void* w
     case 2: st = launch_wide<2>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, waves, halves, direct, out_stride, out_f32, nl, stream); break;
     case 3: st = launch_wide<3>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, waves, halves, direct, out_stride, out_f32, nl, stream); break;
     case 4: st = launch_wide<4>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, nt, waves, halves, direct, out_stride, out_f32, nl, stream); break;
-    case 5: st = launch_wide_tall<5>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
-    case 6: st = launch_wide_tall<6>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
-    case 7: st = launch_wide_tall<7>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
-    default: st = launch_wide_tall<8>(part, (const bf16_t*)x, (const bf16_t*)wt, M, N, K, x_stride, ksplit, direct, out_stride, out_f32, stream); break;
+    case 5: st = launch_wide_tall<5>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, waves, halves, direct, out_stride, out_f32, stream); break;
+    case 6: st = launch_wide_tall<6>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, waves, halves, direct, out_stride, out_f32, stream); break;
+    case 7: st = launch_wide_tall<7>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, waves, halves, direct, out_stride, out_f32, stream); break;
+    default: st = launch_wide_tall<8>(part, (const bf16_t*)x, (const bf16_t*)wt, (const bf16_t*)wt2, M, N, K, x_stride, ksplit, waves, halves, direct, out_stride, out_f32, stream); break;
   }
   if (st != NS_OK || direct) return st;
   if (defer) return epi == 0 ? NS_OK : NS_ERR_BAD_ARG;
@@ -380,7 +389,7 @@ extern "C" int ns_gemm_wide_bf16(void* out, void* workspace, const void* x, cons
 
 // The same with the number of waves per workgroup and the unit of work chosen by the caller (see wide_product), so that
 // the row tiles can be dealt evenly to the compute units, and with the partial sums of a norm before the product (ssq_in may
-// be null; see WideNorm).
+// be null; see WideNorm).  halves: up to 128 rows.
 extern "C" int ns_gemm_wide_dealt_bf16(void* out, void* workspace, const void* x, const void* wt, const void* wt2, int M, int N,
                                        int K, int x_stride, int out_stride, int epi, int out_f32, int ksplit, int nt, int defer,
                                        int waves, int halves, const float* ssq_in, int parts_in, int norm_dim, float eps,

@@ -451,10 +451,12 @@ def wide_waves(n: int, k: int, rows: int, ksplit: int, nt: int, gated: bool = Fa
     seven or four waves of half a tile of each (7 or 4 a workgroup); at the 8B shape 1,792 half tiles are 7 for each of 256
     units instead of 8 for each of 224 (42 against 51 us at 64 rows; the 1B shape's 1,024 as 4 for each: 17 against 25 us)."""
     units = units or compute_units(torch.cuda.current_device())
-    if rows > SKINNY_MAX_ROWS or nt != 1:
+    if nt != 1 or (rows > SKINNY_MAX_ROWS and not gated):
         return 4, False
     tiles, k_tiles = -(-n // 16), -(-k // 128)
     if gated:
+        if rows > SKINNY_MAX_ROWS:  # 65 to 128 rows: only half tiles hold the sums of both matrices
+            return (7 if -(-(-(-2 * tiles // 7)) // units) * 7 <= -(-(-(-2 * tiles // 4)) // units) * 4 else 4), ksplit == 1
         if ksplit != 1 or -(-tiles // 4) >= units:  # (whole tiles fill the GPU: measured level or ahead, 163 against 166 us at the 70B shape)
             return 4, False
         options = [(-(-(-(-tiles // 4)) // units) * 8, 4, False), (-(-(-(-2 * tiles // 7)) // units) * 7, 7, True),
@@ -486,8 +488,12 @@ def linear_wide(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight |
     want = torch.float32 if out_f32 else x.dtype
     plan = wide_plan(w.n, w.k, m)
     ksplit, nt = ksplit or plan[0], nt or plan[1]
-    if m > SKINNY_MAX_ROWS and (w2 is not None or nt != 1):
-        raise KernelRefused(f"linear_wide takes more than {SKINNY_MAX_ROWS} rows only for one matrix with one row tile per wave")
+    if not waves:
+        waves, dealt_halves = wide_waves(w.n, w.k, m, ksplit, nt, gated=w2 is not None)
+        halves = dealt_halves if halves is None else halves
+    halves = bool(halves)
+    if m > SKINNY_MAX_ROWS and ((w2 is not None and not halves) or nt != 1):
+        raise KernelRefused(f"linear_wide takes more than {SKINNY_MAX_ROWS} rows only with one row tile per wave, and two matrices only by half tiles")
     defer = defer and ksplit > 1 and w2 is None and not out_f32
     if out is None and not defer:
         out = torch.empty((m, w.n), dtype=want, device=x.device)
@@ -500,14 +506,10 @@ def linear_wide(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight |
         workspace = torch.empty(need, dtype=torch.float32, device=x.device)
     if need and (workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous()):
         raise KernelRefused("linear_wide: workspace too small")
-    if not waves:
-        waves, dealt_halves = wide_waves(w.n, w.k, m, ksplit, nt, gated=w2 is not None)
-        halves = dealt_halves if halves is None else halves
-    halves = bool(halves)
     if pre is not None and (ksplit != 1 or defer):
         raise KernelRefused("linear_wide: a pre-normed input goes with one range of K")
-    if halves and (w2 is None or ksplit != 1 or nt != 1 or m > SKINNY_MAX_ROWS or waves not in (4, 7)):
-        raise KernelRefused("linear_wide: half tiles go with two matrices, one range, one tile per wave, up to 64 rows, 4 or 7 waves")
+    if halves and (w2 is None or ksplit != 1 or nt != 1 or waves not in (4, 7)):
+        raise KernelRefused("linear_wide: half tiles go with two matrices, one range, one tile per wave, 4 or 7 waves")
     if not halves and waves != 4 and not (waves == 3 and w2 is None and nt == 1 and m <= SKINNY_MAX_ROWS):
         raise KernelRefused("linear_wide: workgroups of 4 waves, or of 3 for one matrix with one tile per wave and up to 64 rows")
     _check(build.core().ns_gemm_wide_dealt_bf16(_ptr(None if defer else out), _ptr(workspace if need else None), _ptr(x), _ptr(w.data),

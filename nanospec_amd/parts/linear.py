@@ -27,6 +27,7 @@ LAYOUTS = ("both", "tiled")
 
 
 STREAM_ROWS = 16  # up to here the streaming kernel beats the library at the shapes measured
+GATED_WIDE_ROWS = 80  # up to here gate and up with the activation go through the 17-to-128-row kernel where the library's layout is kept too
 WIDE_HEAD_ROWS = 12  # above this many rows a wide 32-bit product (the head) is faster through the 17-to-64-row kernel
 WIDE_MAX_N = 4096  # 17 to 64 rows: the hand-written kernel is ahead of the library for outputs up to this width (and for
 #                    32-bit results, which the library does not give); wider products go to the library
@@ -242,11 +243,14 @@ class GatedWeights:
         if fast and stacked is None and m > ops.WIDE_TALL_ROWS:
             # only the tiled layout is kept: blocks of 128 rows through the hand-written kernel, activation in the same pass
             return ops.linear_rows(x, self.tiled[0], w2=self.tiled[1], out=out, ksplit=1, nt=2)
-        if fast and (m <= ops.SKINNY_MAX_ROWS or stacked is None):
-            # 17 to 64 rows: the second hand-written kernel, one range of K, so that the activation is applied in the same
-            # pass (measured ahead of the library's product plus the activation kernel)
-            for s in range(0, m, ops.SKINNY_MAX_ROWS):
-                e = min(m, s + ops.SKINNY_MAX_ROWS)
+        if fast and (m <= GATED_WIDE_ROWS or stacked is None):
+            # 17 to 80 rows: the second hand-written kernel, one range of K, so that the activation is applied in the same
+            # pass (measured ahead of the library's product plus the activation kernel: 50 against 60 us at 72 rows of the
+            # 8B shape, level at 96).  Beyond 64 rows it holds the sums of both matrices only by half tiles; where only the
+            # tiled layout is kept it takes up to 128 rows a pass that way (70B shape: 243 us where two passes of 64 take 331).
+            step = ops.WIDE_TALL_ROWS if ops.wide_waves(self.inter, self.k, ops.WIDE_TALL_ROWS, 1, 1, gated=True)[1] else ops.SKINNY_MAX_ROWS
+            for s in range(0, m, step):
+                e = min(m, s + step)
                 ops.linear_wide(x[s:e], self.tiled[0], w2=self.tiled[1], out=out[s:e], ksplit=1, nt=1)
             return out
         gu = ctx.arena.take((m, 2 * self.inter), x.dtype)

@@ -198,7 +198,9 @@ def test_wide_plans_deal_evenly():
     assert ops.wide_waves(14336, 4096, 64, 1, 1, gated=True, units=256) == (7, True)   # 1,792 half tiles: 7 for each of 256 units
     assert ops.wide_waves(8192, 2048, 64, 1, 1, gated=True, units=256) == (4, True)    # 1,024 half tiles: 4 for each
     assert ops.wide_waves(28672, 8192, 64, 1, 1, gated=True, units=256) == (4, False)  # 448 workgroups of whole tiles fill the GPU
-    assert ops.wide_waves(14336, 4096, 100, 1, 1, units=256) == (4, False)             # more than 64 rows: four waves
+    assert ops.wide_waves(14336, 4096, 100, 1, 1, units=256) == (4, False)             # more than 64 rows of one matrix: four waves
+    assert ops.wide_waves(14336, 4096, 100, 1, 1, gated=True, units=256) == (7, True)  # gate and up: half tiles only
+    assert ops.wide_waves(8192, 2048, 100, 1, 1, gated=True, units=256) == (4, True)
     assert ops.wide_waves(14336, 4096, 64, 2, 1, gated=True, units=256) == (4, False)  # gate and up over ranges: whole tiles
 
 
@@ -459,9 +461,18 @@ def test_linear_wide_up_to_128_rows(m, n, k):
     with pytest.raises(ops.KernelRefused):
         ops.linear_wide(x, wt, nt=2)
     with pytest.raises(ops.KernelRefused):
-        ops.linear_wide(x, wt, w2=wt)
+        ops.linear_wide(x, wt, w2=wt, ksplit=1, nt=1, waves=4, halves=False)  # whole tiles of two matrices: up to 64 rows
     with pytest.raises(ops.KernelRefused):
         ops.linear_wide(torch.randn(129, k, dtype=torch.bfloat16, device=DEV), wt)
+    # gate and up by half tiles hold one set of sums, so they take these rows too
+    w2 = torch.randn(n, k, dtype=torch.bfloat16, device=DEV)
+    wt2 = ops.TiledWeight(w2)
+    want = ref * torch.sigmoid(ref) * (x.cpu().float() @ w2.cpu().float().T)
+    seven = ops.linear_wide(x, wt, w2=wt2, ksplit=1, nt=1, waves=7, halves=True)
+    assert ulps_of_row_max(seven.cpu(), want).max() <= 1.0
+    assert torch.equal(ops.linear_wide(x, wt, w2=wt2, ksplit=1, nt=1, waves=4, halves=True), seven)
+    assert torch.equal(ops.linear_wide(x, wt, w2=wt2, ksplit=1, nt=1), seven)  # (the form the plan deals: one of the two)
+    assert torch.equal(seven[:64], ops.linear_wide(x[:64], wt, w2=wt2, ksplit=1, nt=1, waves=4, halves=False))
 
 
 @pytest.mark.parametrize("m", [129, 300, 1031])
