@@ -246,9 +246,9 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       for (int t = 0; t < 2 * CT; ++t) o[t % CT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_piece(at, t), pf[t / CT], o[t % CT], 0, 0, 0);
     };
 
-    // Before round 0: the keys of blocks 0, 1 and 2 and the values of blocks 0 and 1 are in their ring buffers, the
+    // Before the first round: the keys of blocks 0, 1 and 2 and the values of blocks 0 and 1 are in their ring buffers, the
     // scores of block 0 are formed, and the page ids of blocks 3 and 2 are at hand for the keys and the values that
-    // round 0 asks for.
+    // first round asks for.
     int ids_k[PPB], ids_v[PPB];
     {
       const int nb = kb1 - kb0;
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       }
       if (nb > 2) load_k(ids_v, kb0 + 2, 2);
     }
-    // (loads land in the order they were asked for: the first scores wait for the keys of block 0 only, round 0 for the
+    // (loads land in the order they were asked for: the first scores wait for the keys of block 0 only, the first round for the
     // values of block 0 and the keys of block 1; a range of fewer than three blocks waits for all it asked for)
     if (kb1 - kb0 > 2)
       NS_WAIT_LOADS(4 * IPW);
