@@ -19,6 +19,7 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
 from pathlib import Path
 
@@ -33,18 +34,27 @@ ATTN_SOURCES = ["attn_mfma.hip"]
 _loaded: dict[str, ctypes.CDLL] = {}
 
 
+_build_dir_found: Path | None = None
+_build_dir_lock = threading.Lock()
+
+
 def _build_dir() -> Path:
-    d = CSRC / "_build"
-    try:
-        d.mkdir(exist_ok=True)
-        probe = d / f".w{os.getpid()}"
-        probe.write_text("")
-        probe.unlink()
-        return d
-    except OSError:
-        d = Path(tempfile.gettempdir()) / f"nanospec_amd_build_{os.getuid()}"
-        d.mkdir(parents=True, exist_ok=True)
-        return d
+    """Where libraries are built: beside the sources, or a per-user temporary folder if that cannot be written.  Found
+    once per process (several compilers run at a time, and all of them must land in the same place)."""
+    global _build_dir_found
+    with _build_dir_lock:
+        if _build_dir_found is None:
+            d = CSRC / "_build"
+            try:
+                d.mkdir(exist_ok=True)
+                probe = d / f".w{os.getpid()}"
+                probe.write_text("")
+                probe.unlink()
+            except OSError:
+                d = Path(tempfile.gettempdir()) / f"nanospec_amd_build_{os.getuid()}"
+                d.mkdir(parents=True, exist_ok=True)
+            _build_dir_found = d
+        return _build_dir_found
 
 
 def _hipcc() -> str:
