@@ -215,8 +215,11 @@ class GatedWeights:
     def _few_rows(self, x, m: int, out: torch.Tensor) -> torch.Tensor:
         """Up to 16 rows (plain or pre-normed).  From a few rows on, where the number of row tiles deals unevenly to the
         compute units as whole tiles, the kernel that shares x through LDS and takes half tiles is ahead of the one that
-        streams a tile per workgroup (8B shape: 37.6 against 39.7 us at 8 rows, 37.4 against 43.8 at 16)."""
-        if m > ops.GATED_HALF_ROWS and ops.wide_waves(self.inter, self.k, m, 1, 1, gated=True)[1]:
+        streams a tile per workgroup (8B shape, 896 tiles on 256 units: 37.6 against 39.7 us at 8 rows, 37.4 against 43.8
+        at 16); where the tiles deal evenly it is not (1B shape, 512 tiles: 2% of a decode step behind)."""
+        tiles, units = -(-self.inter // 16), ops.compute_units(out.device)
+        uneven = -(-tiles // units) * units > 1.05 * tiles  # a tile of each matrix per workgroup leaves some units a round short
+        if m > ops.GATED_HALF_ROWS and uneven and ops.wide_waves(self.inter, self.k, m, 1, 1, gated=True, units=units)[1]:
             return ops.linear_wide(x, self.tiled[0], w2=self.tiled[1], out=out, ksplit=1, nt=1)
         return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
 
