@@ -32,22 +32,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 // compute unit with the most workgroups, and 14,336 rows are 3.5 workgroups per compute unit of the one kind (as slow as 4)
 // and 7 of the other.
 
-// What the q/k/v epilogue needs: the rows of the stacked [q; k; v] matrix were permuted at load time so that a
-// workgroup's 16 rows are, for the rotary part of a q or k head, the first channels of 8 pairs j and then their second
-// channels (rope.h: j and j + rot/2, or 2j and 2j + 1), and otherwise 16 consecutive channels.  The epilogue rotates
-// (rope.h), writes q into
-// the attention input, k into its K page slot and v into the transposed V page
-// (reference: model/llama.py:175-183; kv/cache.py:23-26).
-struct RopeKvParams {
-  const int* positions;    // [M]
-  const int* token_req;    // [M]
-  const int* block_table;  // [requests, table_stride]
-  const float* inv_freq;   // [rot / 2]
-  bf16_t* k_cache;         // [pages, kv_heads, page, hd]
-  bf16_t* v_cache;         // [pages, kv_heads, hd, page]
-  int table_stride, heads, kv_heads, hd, rot, page_size, write_kv;
-  RopeForm form;           // rot again, the pairing and the factor on cosine and sine
-};
+// (RopeKvParams, what the q/k/v epilogue needs, and the epilogue's work for one pair of sums: rope.h)
 
 // How a product can take over the work of the norm kernels around it (reference for the norm: model/llama.py:86-95, for
 // the sums it sits between: model/llama.py:198-208).  RMS norm is y = w * (r / rms(r)); the division is a factor per
@@ -205,9 +190,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
     // thread e <-> (token m, pair p): the sums of local rows p and p + 8
     const int tiles_per_head = rk.hd / 16;
     const int gh = blockIdx.x / tiles_per_head, jt = blockIdx.x % tiles_per_head;  // head among [q heads | k heads | v heads]
-    const bool is_q = gh < rk.heads, is_v = gh >= rk.heads + rk.kv_heads;
-    const int rot_tiles = is_v ? 0 : rk.rot / 16;
-    const bool rotary = jt < rot_tiles;
     for (int e = threadIdx.x; e < M * 8; e += WAVES * 64) {
       const int m = e >> 3, p = e & 7;
       const int mt = m >> 4, mr = m & 15;
@@ -223,37 +205,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
         x1 *= rinv_s[m];
         x2 *= rinv_s[m];
       }
-      int d1, d2;
-      if (rotary) {
-        const int j = jt * 8 + p;
-        float c, sn;
-        rope_cos_sin(rk.form, rk.positions[m], rk.inv_freq[j], c, sn);
-        rope_turn(x1, x2, c, sn, x1, x2);
-        rope_pair_channels(rk.form, j, d1, d2);
-      } else {
-        d1 = rk.rot * (is_v ? 0 : 1) + (jt - rot_tiles) * 16 + p;
-        d2 = d1 + 8;
-      }
-      if (is_q) {
-        bf16_t* o = (bf16_t*)out + (size_t)m * out_stride + gh * rk.hd;
-        o[d1] = (bf16_t)x1;
-        o[d2] = (bf16_t)x2;
-      } else if (rk.write_kv) {
-        const int pos = rk.positions[m];
-        const int page = rk.block_table[(size_t)rk.token_req[m] * rk.table_stride + pos / rk.page_size];
-        const int off = pos % rk.page_size;
-        if (!is_v) {
-          const int kh = gh - rk.heads;
-          bf16_t* kd = rk.k_cache + (((size_t)page * rk.kv_heads + kh) * rk.page_size + off) * rk.hd;
-          kd[d1] = (bf16_t)x1;
-          kd[d2] = (bf16_t)x2;
-        } else {
-          const int vh = gh - rk.heads - rk.kv_heads;
-          bf16_t* vd = rk.v_cache + (((size_t)page * rk.kv_heads + vh) * rk.hd) * rk.page_size + off;
-          vd[(size_t)d1 * rk.page_size] = (bf16_t)x1;
-          vd[(size_t)d2 * rk.page_size] = (bf16_t)x2;
-        }
-      }
+      rope_kv_store_pair(rk, out, out_stride, m, gh, jt, p, x1, x2);
     }
     return;
   }
