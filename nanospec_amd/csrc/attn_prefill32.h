@@ -165,7 +165,7 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
     // inside the held pages: a key outside [wlo, whi) is masked anyway, and so any block may be asked for.
     typedef const __attribute__((address_space(4))) int* scalar_ints;
     const scalar_ints stable = (scalar_ints)(unsigned long long)table;
-    const int lo_slot = wlo >> psh, hi_slot = (whi - 1) >> psh;
+    const int lo_slot = wlo >> psh, hi_slot = max((whi - 1) >> psh, lo_slot);  // (a tile without tokens sees no key: slot 0 of its row)
     auto page_ids = [&](int(&ids)[PPB], int kb) {
       const int first = (kb * 32) >> psh;
 #pragma unroll

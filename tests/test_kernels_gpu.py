@@ -658,7 +658,7 @@ def test_untile_gives_the_matrix_back(n, k):
 
 
 def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force_splits=None, qt=2, coop=False, step_keys=0,
-              chunk_splits=1, short_offsets=True):
+              chunk_splits=1, short_offsets=True, spare_tiles=0):
     n = sum(lens)
     indptr = [0]
     for l in lens:
@@ -667,6 +667,7 @@ def _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, window=0, force
     group = heads // kvh
     tile = lambda b, t0: [b, t0, indptr[b], lens[b], starts[b] + lens[b], 0, 0, 0]
     ct = [tile(b, t0) for b, l in enumerate(lens) if l != 1 for t0 in range(0, l, 16 * qt)]
+    ct += [[len(lens) - 1, 0, 0, 0, 0, 0, 0, 0]] * (spare_tiles if ct else 0)  # tiles without tokens, as a captured step's spare ones
     dt = [tile(b, 0) for b, l in enumerate(lens) if l == 1]
     for t in dt:
         t[5] = step_keys  # the keys all decode rows of the step read: from some number on the kernel reads them past the cache
@@ -735,7 +736,8 @@ def test_attention_mfma_prompt_kernel_page_sizes_and_groups(case, heads, kvh, hd
     q = torch.randn(n, heads * hd, dtype=torch.bfloat16, device=DEV)
     ref = plain_paged_attention(q.view(n, heads, hd), kvs, starts, lens, heads).reshape(n, -1)
     for coop, chunk_splits in ((False, 1), (True, 1), (True, 3), (False, 16)):
-        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, qt=2, coop=coop, chunk_splits=chunk_splits, short_offsets=short_offsets)
+        out = _run_mfma(ops, q, k, v, table, starts, lens, heads, kvh, hd, qt=2, coop=coop, chunk_splits=chunk_splits, short_offsets=short_offsets,
+                        spare_tiles=3 if chunk_splits in (1, 3) else 0)
         u = ulps_of_row_max(out.cpu(), ref).max()
         assert u <= 4, f"{case} coop={coop} chunk_splits={chunk_splits}: {u:.2f} ulps"
 
